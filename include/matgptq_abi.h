@@ -1,0 +1,127 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of MatGPTQ's bit-sliced GEMM.
+ *
+ * Plain pointers and sizes only; no torch types.  Every function returns 0 on
+ * success or a negative MATGPTQ_E* code (never exits the process, never
+ * synchronises the device unless the SYNC convention below asks for it).
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ * Pointers named *_dev are device memory, *_host are host memory.
+ *
+ * Naming of sizes follows torch.nn.Linear: W is [N, K] (out x in), X is [M, K],
+ * Y = X * W^T is [M, N].  The reference calls them m (=N), n (=K), k (=M).
+ *
+ * Preconditions shared by all entry points: bitwidth in {2,3,4,6,8},
+ * group_size in {-1,32,128}, N % 16 == 0, K % 128 == 0.
+ */
+#ifndef MATGPTQ_ABI_H
+#define MATGPTQ_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MATGPTQ_ABI_VERSION 1
+
+/* error codes */
+#define MATGPTQ_OK 0
+#define MATGPTQ_EBITS (-1)     /* bitwidth not in {2,3,4,6,8} */
+#define MATGPTQ_EGROUP (-2)    /* group_size not in {-1,32,128} or does not divide K */
+#define MATGPTQ_ESHAPE (-3)    /* N % 16 != 0, K % 128 != 0, or a size <= 0 */
+#define MATGPTQ_ENULL (-4)     /* a required pointer is NULL */
+#define MATGPTQ_EDTYPE (-5)    /* bf16 requested (flag bit 1): not built yet */
+#define MATGPTQ_ELAUNCH (-6)   /* the HIP runtime reported an error at launch */
+#define MATGPTQ_EVARIANT (-7)  /* a forced kernel variant does not apply to this problem */
+#define MATGPTQ_ESIZE (-8)     /* a size exceeds what the entry point supports */
+
+/* feature_flag bits: the reference's `Features` word
+ * (inference_lib/matgptq_cuda/csrc/include/common.cuh:78-86,
+ *  inference_lib/matgptq_cuda/matgptq_linear.py:6-9). */
+#define MATGPTQ_FLAG_ASYNC 1u /* bit 0: 1 = do not synchronise after the launch */
+#define MATGPTQ_FLAG_BF16 2u  /* bit 1: activations / scales / output are bf16 */
+/* Bits 8..15: benchmark-only override of the kernel variant (0 = automatic). */
+#define MATGPTQ_FLAG_VARIANT_SHIFT 8
+#define MATGPTQ_FLAG_VARIANT_MASK 0xFF00u
+
+int matgptq_abi_version(void);
+const char *matgptq_strerror(int code);
+
+/* Number of uint32 words of a packed weight: bitwidth*N*K/32, the size the
+ * reference's op checks (inference_lib/matgptq_cuda/csrc/bindings.cpp:68,160).
+ * Returns 0 for invalid arguments. */
+size_t matgptq_packed_words(int bitwidth, int64_t N, int64_t K);
+
+/* ---- the GEMM ------------------------------------------------------------
+ * Replaces MATGPTQ_CUDA::matmul_matgptq_host
+ * (inference_lib/matgptq_cuda/csrc/include/gemm.h:22-32,
+ *  inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:1026-1065).
+ *
+ *   Y[M,N] = fp16( sum_k X[m,k] * scale[n,k/g] * ((c[n,k] << (8-b)) - zero[n,k/g]) )
+ *
+ * packed_dev   output of matgptq_pack_* (b-bit codes c, already sliced)
+ * scales_dev   output of matgptq_reorder_scales_* applied to scale[N, K/g] (fp16)
+ * zeros_dev    output of matgptq_reorder_scales_* applied to zero[N, K/g] (fp16),
+ *              or NULL: every zero is 128, which is the reference kernel's
+ *              symmetric form  (c - 2^(b-1)) * scale * 2^(8-b)
+ * x_dev        [M, K] fp16 row-major;  y_dev  [M, N] fp16 row-major
+ * Any M >= 1 is accepted.  Graph-capturable: no allocation, no host read.
+ * With flag bit 0 clear the call ends with hipStreamSynchronize(stream). */
+int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                 const void *packed_dev, const void *scales_dev, const void *zeros_dev,
+                 const void *x_dev, void *y_dev, void *stream, uint32_t flags);
+
+/* ---- packing on the host ---------------------------------------------------
+ * Replaces swizzle_weights / split_up_n_bits / swizzle_matgptq
+ * (inference_lib/matgptq_cuda/csrc/utils.cpp:22-217) as driven by
+ * pack_matgptq_qweights (inference_lib/matgptq_cuda/csrc/bindings.cpp:43-84).
+ * codes_host: uint8 [N, K].  If slice_from_master != 0 the codes are 8-bit
+ * master codes and are first sliced to `bitwidth` with the reference's rounded
+ * slice (src/quant_utils_matgpqt.py:9-17); otherwise they must already be
+ * < 2^bitwidth (higher bits are ignored).  out_host: matgptq_packed_words() words. */
+int matgptq_pack_host(const uint8_t *codes_host, int64_t N, int64_t K, int bitwidth,
+                      int slice_from_master, uint32_t *out_host);
+
+/* Inverse of matgptq_pack_host (tests, bit-exactness checks). */
+int matgptq_unpack_host(const uint32_t *packed_host, int64_t N, int64_t K, int bitwidth,
+                        uint8_t *codes_host);
+
+/* Replaces reorder_matgptq_scales (inference_lib/matgptq_cuda/csrc/bindings.cpp:86-142).
+ * in: 16-bit elements [N, G] (G = K/g, 1 for g = -1); out: same count, ordered
+ * [N/16][G][16] so that the 16 rows of a tile are contiguous per group.
+ * Works on any 16-bit type (fp16 scales, fp16 zeros, bf16). */
+int matgptq_reorder_scales_host(const uint16_t *in_host, int64_t N, int64_t K, int group_size,
+                                uint16_t *out_host);
+
+/* ---- packing on the device ---------------------------------------------------
+ * Same results as the host functions, for tensors that already live in HBM
+ * (the reference copies to the host and back, bindings.cpp:70-83,99-141).
+ * Asynchronous on `stream`. */
+int matgptq_pack_device(const uint8_t *codes_dev, int64_t N, int64_t K, int bitwidth,
+                        int slice_from_master, uint32_t *out_dev, void *stream);
+int matgptq_unpack_device(const uint32_t *packed_dev, int64_t N, int64_t K, int bitwidth,
+                          uint8_t *codes_dev, void *stream);
+int matgptq_reorder_scales_device(const uint16_t *in_dev, int64_t N, int64_t K, int group_size,
+                                  uint16_t *out_dev, void *stream);
+
+/* Rounded MSB slice of master codes on the device, element-wise
+ * (src/quant_utils_matgpqt.py:9-17 with master_bitwidth = 8). */
+int matgptq_slice_device(const uint8_t *master_dev, int64_t count, int bitwidth,
+                         uint8_t *sliced_dev, void *stream);
+
+/* Dequantised weight W[N,K] (fp16) from a packed tensor, rounded once per
+ * element exactly like the reference's dequantize (src/quant_utils_matgpqt.py:19-22).
+ * Used by tests and by callers that want a dense copy. */
+int matgptq_dequantize_device(int bitwidth, int group_size, int64_t N, int64_t K,
+                              const void *packed_dev, const void *scales_dev,
+                              const void *zeros_dev, void *w_dev, void *stream);
+
+/* Human-readable name of the kernel variant matgptq_gemm would launch. */
+int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                          int has_zeros, uint32_t flags, char *buf, size_t buf_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MATGPTQ_ABI_H */

@@ -1,0 +1,238 @@
+// C ABI entry points: argument checks, kernel selection, launches.
+// Counterpart of the reference's host launcher and dispatch macros
+// (inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:955-1065); it returns error
+// codes where the reference prints and exits (include/common.cuh:44-51).
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/matgptq_abi.h"
+#include "device_common.h"
+
+namespace matgptq {
+
+int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host.cpp
+
+#define MATGPTQ_DECL(B)                                                                        \
+  hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int W, bool xlds,      \
+                                hipStream_t);                                                  \
+  hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);
+MATGPTQ_DECL(2)
+MATGPTQ_DECL(3)
+MATGPTQ_DECL(4)
+MATGPTQ_DECL(6)
+MATGPTQ_DECL(8)
+#undef MATGPTQ_DECL
+
+hipError_t launch_pack(const uint8_t*, int64_t, int64_t, int, int, uint32_t*, hipStream_t);
+hipError_t launch_unpack(const uint32_t*, int64_t, int64_t, int, uint8_t*, hipStream_t);
+hipError_t launch_slice(const uint8_t*, int64_t, int, uint8_t*, hipStream_t);
+hipError_t launch_reorder(const uint16_t*, int64_t, int64_t, uint16_t*, hipStream_t);
+hipError_t launch_dequant(int, int, int64_t, int64_t, const uint32_t*, const uint16_t*,
+                          const uint16_t*, uint16_t*, hipStream_t);
+
+namespace {
+
+constexpr int kDecodeMaxM = 16;
+constexpr size_t kLdsBudget = 64 * 1024;  // dynamic LDS a decode workgroup may ask for
+
+struct Plan {
+  bool decode;
+  int R, W;      // decode: row blocks per workgroup, waves per workgroup
+  bool xlds;     // decode: activations staged in LDS
+  int cfg;       // prefill: tile configuration
+};
+
+int largest_r(int want, int row_blocks) {
+  int r = want;
+  while (r > 1 && row_blocks % r != 0) r >>= 1;
+  return r;
+}
+
+// Automatic choice; `variant` (flags bits 8..15) overrides it for benchmarks:
+//   decode : 1 + rsel + 3*wsel + 9*xsel,  rsel: R = 1,2,4   wsel: W = 2,4,8   xsel: 0 global, 1 LDS
+//   prefill: 64 + cfg
+int make_plan(int bits, int64_t N, int64_t K, int64_t M, uint32_t flags, Plan* p) {
+  const int row_blocks = (int)(N / 16), k_tiles = (int)(K / 128);
+  const int variant = (int)((flags & MATGPTQ_FLAG_VARIANT_MASK) >> MATGPTQ_FLAG_VARIANT_SHIFT);
+  p->decode = M <= kDecodeMaxM;
+  p->cfg = 0;
+  // default decode shape
+  int W = k_tiles >= 32 ? 8 : (k_tiles >= 8 ? 4 : 2);
+  int R = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
+  while (R > 1 && row_blocks / R < 512) R >>= 1;  // keep the grid wide
+  R = largest_r(R, row_blocks);
+  bool xlds = true;
+  // default prefill tile: wide tiles for big problems, narrow ones otherwise
+  if (!p->decode) {
+    if (M <= 32) p->cfg = 4;
+    else if (M <= 64) p->cfg = 2;
+    else p->cfg = 0;
+  }
+  if (variant != 0) {
+    if (variant >= 64) {
+      if (variant - 64 > 4 || M < 1) return MATGPTQ_EVARIANT;
+      p->decode = false;
+      p->cfg = variant - 64;
+    } else {
+      if (M > kDecodeMaxM) return MATGPTQ_EVARIANT;
+      const int v = variant - 1;
+      if (v >= 18) return MATGPTQ_EVARIANT;
+      p->decode = true;
+      R = 1 << (v % 3);
+      W = 2 << ((v / 3) % 3);
+      xlds = (v / 9) != 0;
+      if (row_blocks % R != 0) return MATGPTQ_EVARIANT;
+    }
+  }
+  const size_t lds = (size_t)W * R * 1024 + (size_t)M * (K + 8) * 2;
+  if (xlds && lds > kLdsBudget) {
+    if (variant != 0 && variant < 64) return MATGPTQ_EVARIANT;
+    xlds = false;
+  }
+  p->R = R;
+  p->W = W;
+  p->xlds = xlds;
+  (void)bits;
+  return MATGPTQ_OK;
+}
+
+hipError_t launch_decode(int bits, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+  switch (bits) {
+    case 2: return launch_decode_b2(a, g, p.R, p.W, p.xlds, s);
+    case 3: return launch_decode_b3(a, g, p.R, p.W, p.xlds, s);
+    case 4: return launch_decode_b4(a, g, p.R, p.W, p.xlds, s);
+    case 6: return launch_decode_b6(a, g, p.R, p.W, p.xlds, s);
+    default: return launch_decode_b8(a, g, p.R, p.W, p.xlds, s);
+  }
+}
+
+hipError_t launch_prefill(int bits, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+  switch (bits) {
+    case 2: return launch_prefill_b2(a, g, p.cfg, s);
+    case 3: return launch_prefill_b3(a, g, p.cfg, s);
+    case 4: return launch_prefill_b4(a, g, p.cfg, s);
+    case 6: return launch_prefill_b6(a, g, p.cfg, s);
+    default: return launch_prefill_b8(a, g, p.cfg, s);
+  }
+}
+
+}  // namespace
+}  // namespace matgptq
+
+using namespace matgptq;
+
+extern "C" {
+
+int matgptq_abi_version(void) { return MATGPTQ_ABI_VERSION; }
+
+const char* matgptq_strerror(int code) {
+  switch (code) {
+    case MATGPTQ_OK: return "ok";
+    case MATGPTQ_EBITS: return "bitwidth must be one of {2, 3, 4, 6, 8}";
+    case MATGPTQ_EGROUP: return "group_size must be one of {-1, 32, 128} and divide n_in_features";
+    case MATGPTQ_ESHAPE: return "n_out_features must be a multiple of 16 and n_in_features a multiple of 128";
+    case MATGPTQ_ENULL: return "null pointer argument";
+    case MATGPTQ_EDTYPE: return "bfloat16 is not supported by this build";
+    case MATGPTQ_ELAUNCH: return "HIP launch failed";
+    case MATGPTQ_EVARIANT: return "forced kernel variant does not apply to this problem";
+    case MATGPTQ_ESIZE: return "size exceeds the supported maximum";
+    default: return "unknown error";
+  }
+}
+
+int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                 const void* packed_dev, const void* scales_dev, const void* zeros_dev,
+                 const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
+  if (int e = check_problem(bitwidth, group_size, N, K)) return e;
+  if (M <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return MATGPTQ_ESIZE;
+  if (!packed_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
+  if (flags & MATGPTQ_FLAG_BF16) return MATGPTQ_EDTYPE;
+  Plan p;
+  if (int e = make_plan(bitwidth, N, K, M, flags, &p)) return e;
+  GemmArgs a;
+  a.packed = static_cast<const uint32_t*>(packed_dev);
+  a.scales = static_cast<const uint16_t*>(scales_dev);
+  a.zeros = static_cast<const uint16_t*>(zeros_dev);
+  a.x = static_cast<const uint16_t*>(x_dev);
+  a.y = static_cast<uint16_t*>(y_dev);
+  a.N = (int)N;
+  a.K = (int)K;
+  a.M = (int)M;
+  a.G = group_size == -1 ? 1 : (int)(K / group_size);
+  a.k_tiles = (int)(K / 128);
+  a.row_blocks = (int)(N / 16);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const hipError_t err = p.decode ? launch_decode(bitwidth, a, group_size, p, s)
+                                  : launch_prefill(bitwidth, a, group_size, p, s);
+  if (err != hipSuccess) return MATGPTQ_ELAUNCH;
+  if (!(flags & MATGPTQ_FLAG_ASYNC)) {
+    if (hipStreamSynchronize(s) != hipSuccess) return MATGPTQ_ELAUNCH;
+  }
+  return MATGPTQ_OK;
+}
+
+int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                          int has_zeros, uint32_t flags, char* buf, size_t buf_len) {
+  if (int e = check_problem(bitwidth, group_size, N, K)) return e;
+  if (!buf || buf_len == 0) return MATGPTQ_ENULL;
+  if (M <= 0) return MATGPTQ_ESIZE;
+  Plan p;
+  if (int e = make_plan(bitwidth, N, K, M, flags, &p)) return e;
+  if (p.decode)
+    snprintf(buf, buf_len, "decode b%d g%d zp%d R%d W%d %s", bitwidth, group_size, has_zeros ? 1 : 0,
+             p.R, p.W, p.xlds ? "xlds" : "xglobal");
+  else
+    snprintf(buf, buf_len, "prefill b%d g%d zp%d cfg%d", bitwidth, group_size, has_zeros ? 1 : 0,
+             p.cfg);
+  return MATGPTQ_OK;
+}
+
+int matgptq_pack_device(const uint8_t* codes_dev, int64_t N, int64_t K, int bitwidth,
+                        int slice_from_master, uint32_t* out_dev, void* stream) {
+  if (int e = check_problem(bitwidth, -1, N, K)) return e;
+  if (!codes_dev || !out_dev) return MATGPTQ_ENULL;
+  return launch_pack(codes_dev, N, K, bitwidth, slice_from_master, out_dev,
+                     static_cast<hipStream_t>(stream)) == hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+int matgptq_unpack_device(const uint32_t* packed_dev, int64_t N, int64_t K, int bitwidth,
+                          uint8_t* codes_dev, void* stream) {
+  if (int e = check_problem(bitwidth, -1, N, K)) return e;
+  if (!packed_dev || !codes_dev) return MATGPTQ_ENULL;
+  return launch_unpack(packed_dev, N, K, bitwidth, codes_dev, static_cast<hipStream_t>(stream)) ==
+                 hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+int matgptq_reorder_scales_device(const uint16_t* in_dev, int64_t N, int64_t K, int group_size,
+                                  uint16_t* out_dev, void* stream) {
+  if (int e = check_problem(8, group_size, N, K)) return e;
+  if (!in_dev || !out_dev) return MATGPTQ_ENULL;
+  const int64_t G = group_size == -1 ? 1 : K / group_size;
+  return launch_reorder(in_dev, N, G, out_dev, static_cast<hipStream_t>(stream)) == hipSuccess
+             ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+int matgptq_slice_device(const uint8_t* master_dev, int64_t count, int bitwidth,
+                         uint8_t* sliced_dev, void* stream) {
+  if (!valid_bits(bitwidth)) return MATGPTQ_EBITS;
+  if (count < 0) return MATGPTQ_ESIZE;
+  if (count == 0) return MATGPTQ_OK;
+  if (!master_dev || !sliced_dev) return MATGPTQ_ENULL;
+  return launch_slice(master_dev, count, bitwidth, sliced_dev, static_cast<hipStream_t>(stream)) ==
+                 hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+int matgptq_dequantize_device(int bitwidth, int group_size, int64_t N, int64_t K,
+                              const void* packed_dev, const void* scales_dev,
+                              const void* zeros_dev, void* w_dev, void* stream) {
+  if (int e = check_problem(bitwidth, group_size, N, K)) return e;
+  if (!packed_dev || !scales_dev || !w_dev) return MATGPTQ_ENULL;
+  return launch_dequant(bitwidth, group_size, N, K, static_cast<const uint32_t*>(packed_dev),
+                        static_cast<const uint16_t*>(scales_dev),
+                        static_cast<const uint16_t*>(zeros_dev), static_cast<uint16_t*>(w_dev),
+                        static_cast<hipStream_t>(stream)) == hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+}  // extern "C"
