@@ -41,9 +41,11 @@ extern "C" {
  *  inference_lib/matgptq_cuda/matgptq_linear.py:6-9). */
 #define MATGPTQ_FLAG_ASYNC 1u /* bit 0: 1 = do not synchronise after the launch */
 #define MATGPTQ_FLAG_BF16 2u  /* bit 1: activations / scales / output are bf16 */
-/* Bits 8..15: benchmark-only override of the kernel variant (0 = automatic). */
+/* Bits 8..17: benchmark-only override of the kernel variant (0 = automatic). */
 #define MATGPTQ_FLAG_VARIANT_SHIFT 8
 #define MATGPTQ_FLAG_VARIANT_MASK 0xFF00u
+#define MATGPTQ_FLAG_FLAVOUR_SHIFT 16
+#define MATGPTQ_FLAG_FLAVOUR_MASK 0x30000u
 
 int matgptq_abi_version(void);
 const char *matgptq_strerror(int code);

@@ -15,8 +15,8 @@ namespace matgptq {
 int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host.cpp
 
 #define MATGPTQ_DECL(B)                                                                        \
-  hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int W, bool xlds,      \
-                                hipStream_t);                                                  \
+  hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int S, int W, int kc,  \
+                                int max_wgs, bool stream_flavour, size_t smem, hipStream_t);   \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);
 MATGPTQ_DECL(2)
 MATGPTQ_DECL(3)
@@ -39,72 +39,121 @@ constexpr size_t kLdsBudget = 64 * 1024;  // dynamic LDS a decode workgroup may 
 
 struct Plan {
   bool decode;
-  int R, W;      // decode: row blocks per workgroup, waves per workgroup
-  bool xlds;     // decode: activations staged in LDS
+  int R, S, W;   // decode: row blocks per wave, slots and k-slices per workgroup
+  int kc;        // decode: tiles of K staged in LDS at a time
+  int max_wgs;   // decode: grid cap (0 = none)
+  bool stream;   // decode: double-buffered flavour
+  size_t smem;   // decode: dynamic LDS bytes
   int cfg;       // prefill: tile configuration
 };
 
-int largest_r(int want, int row_blocks) {
-  int r = want;
-  while (r > 1 && row_blocks % r != 0) r >>= 1;
-  return r;
+// (slots, k-slices) per workgroup selectable through the variant override
+constexpr int kNumShapes = 14;
+constexpr int kShapes[kNumShapes][2] = {{1, 8}, {1, 4}, {2, 4}, {2, 2}, {4, 2}, {4, 1}, {8, 1},
+                                        {1, 2}, {2, 1}, {1, 16}, {2, 8}, {4, 4}, {8, 2}, {1, 1}};
+
+// LDS of a decode workgroup: partial sums (1 KiB per wave and row block) and kc tiles
+// of activations.
+size_t decode_lds_bytes(int R, int S, int W, int kc, int64_t M) {
+  return (size_t)S * W * R * 1024 + (size_t)M * ((size_t)kc * 128 + 8) * 2;
 }
 
-// Automatic choice; `variant` (flags bits 8..15) overrides it for benchmarks:
-//   decode : 1 + rsel + 3*wsel + 9*xsel,  rsel: R = 1,2,4   wsel: W = 2,4,8   xsel: 0 global, 1 LDS
-//   prefill: 64 + cfg
-int make_plan(int bits, int64_t N, int64_t K, int64_t M, uint32_t flags, Plan* p) {
+int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
+// Automatic choice; the flags word can override it for benchmarks:
+//   bits 8..15 : 0 = automatic, 1 + rsel + 3*shape = decode (rsel: R = 1,2,4; shape: kShapes),
+//                64 + cfg = prefill tile configuration
+//   bits 16..17: decode flavour, 0 = automatic, 1 = burst, 2 = stream
+//   bits 18..20: decode grid cap, 0 = automatic, 1 = none, n >= 2: (n-1) workgroups per CU
+int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp, uint32_t flags,
+              Plan* p) {
   const int row_blocks = (int)(N / 16), k_tiles = (int)(K / 128);
   const int variant = (int)((flags & MATGPTQ_FLAG_VARIANT_MASK) >> MATGPTQ_FLAG_VARIANT_SHIFT);
+  const int flavour = (int)((flags >> 16) & 3u);
+  const int cap_sel = (int)((flags >> 18) & 7u);
   p->decode = M <= kDecodeMaxM;
   p->cfg = 0;
-  // default decode shape
-  int W = k_tiles >= 32 ? 8 : (k_tiles >= 8 ? 4 : 2);
-  int R = M <= 4 ? 1 : (M <= 8 ? 2 : 4);
-  while (R > 1 && row_blocks / R < 512) R >>= 1;  // keep the grid wide
-  R = largest_r(R, row_blocks);
-  bool xlds = true;
-  // default prefill tile: wide tiles for big problems, narrow ones otherwise
+  // default decode shape (measured on MI355X, M = 1, Llama-3-8B layers): eight waves per
+  // workgroup; few row blocks -> all eight split K, many -> two slots of four k-slices;
+  // two row blocks per wave once there are enough of them to keep the grid wide
+  int W = 8, S = 1;
+  if (row_blocks >= 1024) { W = 4; S = 2; }
+  while (W > 1 && W > k_tiles) { W >>= 1; S <<= 1; }
+  int R = (row_blocks >= 320 && row_blocks % 2 == 0) ? 2 : 1;
+  // default prefill tile
   if (!p->decode) {
     if (M <= 32) p->cfg = 4;
     else if (M <= 64) p->cfg = 2;
-    else p->cfg = 0;
+    else p->cfg = 3;
   }
   if (variant != 0) {
     if (variant >= 64) {
-      if (variant - 64 > 4 || M < 1) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 4) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->cfg = variant - 64;
     } else {
       if (M > kDecodeMaxM) return MATGPTQ_EVARIANT;
       const int v = variant - 1;
-      if (v >= 18) return MATGPTQ_EVARIANT;
+      if (v >= 3 * kNumShapes) return MATGPTQ_EVARIANT;
       p->decode = true;
       R = 1 << (v % 3);
-      W = 2 << ((v / 3) % 3);
-      xlds = (v / 9) != 0;
-      if (row_blocks % R != 0) return MATGPTQ_EVARIANT;
+      S = kShapes[v / 3][0];
+      W = kShapes[v / 3][1];
+      if (W > k_tiles) return MATGPTQ_EVARIANT;
     }
   }
-  const size_t lds = (size_t)W * R * 1024 + (size_t)M * (K + 8) * 2;
-  if (xlds && lds > kLdsBudget) {
-    if (variant != 0 && variant < 64) return MATGPTQ_EVARIANT;
-    xlds = false;
+  if (!p->decode) {
+    p->R = p->S = p->W = p->kc = 0;
+    p->stream = false;
+    p->smem = 0;
+    p->max_wgs = 0;
+    return MATGPTQ_OK;
   }
+  // burst keeps at most eight waves per workgroup; long tile runs prefer stream
+  const int tiles_per_wave = (k_tiles + W - 1) / W * R;
+  bool stream = flavour == 2 || (flavour == 0 && S * W > 8);
+  (void)tiles_per_wave;
+  if (!stream && S * W > 8) return MATGPTQ_EVARIANT;
+  // largest kc whose activations fit next to the partial sums and scales
+  const int64_t fixed = (int64_t)decode_lds_bytes(R, S, W, 0, 0);
+  const int64_t avail = (int64_t)kLdsBudget - fixed;
+  int64_t kc = avail > 0 ? (avail / (2 * M) - 8) / 128 : 0;
+  if (kc < 1) return variant != 0 ? MATGPTQ_EVARIANT : MATGPTQ_ESIZE;
+  if (kc > k_tiles) kc = k_tiles;
+  if (kc >= W) kc = kc / W * W;
   p->R = R;
+  p->S = S;
   p->W = W;
-  p->xlds = xlds;
+  p->kc = (int)kc;
+  p->stream = stream;
+  p->smem = decode_lds_bytes(R, S, W, (int)kc, M);
+  // a capped grid only pays when X' is staged once (kc covers K)
+  p->max_wgs = 0;
+  if (kc >= k_tiles && cap_sel >= 2) p->max_wgs = (cap_sel - 1) * device_cu_count();
+  (void)zp;
+  (void)group_size;
   (void)bits;
   return MATGPTQ_OK;
 }
 
 hipError_t launch_decode(int bits, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
   switch (bits) {
-    case 2: return launch_decode_b2(a, g, p.R, p.W, p.xlds, s);
-    case 3: return launch_decode_b3(a, g, p.R, p.W, p.xlds, s);
-    case 4: return launch_decode_b4(a, g, p.R, p.W, p.xlds, s);
-    case 6: return launch_decode_b6(a, g, p.R, p.W, p.xlds, s);
-    default: return launch_decode_b8(a, g, p.R, p.W, p.xlds, s);
+    case 2: return launch_decode_b2(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
+    case 3: return launch_decode_b3(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
+    case 4: return launch_decode_b4(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
+    case 6: return launch_decode_b6(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
+    default: return launch_decode_b8(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
   }
 }
 
@@ -147,10 +196,12 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
                  const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
   if (int e = check_problem(bitwidth, group_size, N, K)) return e;
   if (M <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return MATGPTQ_ESIZE;
+  // the kernels address the packed tensor with 32-bit byte offsets
+  if ((uint64_t)N * (uint64_t)K / 8 * (uint64_t)bitwidth >= (1ull << 32)) return MATGPTQ_ESIZE;
   if (!packed_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
   if (flags & MATGPTQ_FLAG_BF16) return MATGPTQ_EDTYPE;
   Plan p;
-  if (int e = make_plan(bitwidth, N, K, M, flags, &p)) return e;
+  if (int e = make_plan(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &p)) return e;
   GemmArgs a;
   a.packed = static_cast<const uint32_t*>(packed_dev);
   a.scales = static_cast<const uint16_t*>(scales_dev);
@@ -179,10 +230,11 @@ int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, in
   if (!buf || buf_len == 0) return MATGPTQ_ENULL;
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
-  if (int e = make_plan(bitwidth, N, K, M, flags, &p)) return e;
+  if (int e = make_plan(bitwidth, group_size, N, K, M, has_zeros != 0, flags, &p)) return e;
   if (p.decode)
-    snprintf(buf, buf_len, "decode b%d g%d zp%d R%d W%d %s", bitwidth, group_size, has_zeros ? 1 : 0,
-             p.R, p.W, p.xlds ? "xlds" : "xglobal");
+    snprintf(buf, buf_len, "decode-%s b%d g%d zp%d R%d S%d W%d kc%d cap%d lds%zu",
+             p.stream ? "stream" : "burst", bitwidth, group_size, has_zeros ? 1 : 0, p.R, p.S, p.W,
+             p.kc, p.max_wgs, p.smem);
   else
     snprintf(buf, buf_len, "prefill b%d g%d zp%d cfg%d", bitwidth, group_size, has_zeros ? 1 : 0,
              p.cfg);

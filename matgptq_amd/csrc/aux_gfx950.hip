@@ -58,7 +58,7 @@ unpack_kernel(const uint32_t* __restrict__ packed, uint8_t* __restrict__ codes, 
   auto emit = [&](auto jtag) {
     constexpr int J = decltype(jtag)::value;
     uint32_t raw[4];
-    Codec<BITS>::decode_octet(w, J, raw);
+    raw_octet<BITS, J>(w, raw);
     uint32_t lo = 0, hi = 0;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -117,7 +117,7 @@ dequant_kernel(const uint32_t* __restrict__ packed, const uint16_t* __restrict__
   auto emit = [&](auto jtag) {
     constexpr int J = decltype(jtag)::value;
     uint32_t raw[4];
-    Codec<BITS>::decode_octet(w, J, raw);
+    raw_octet<BITS, J>(w, raw);
     const int64_t k0 = kb * 128 + J * 32 + q * 8;
     const int64_t g = group_size == -1 ? 0 : k0 / group_size;
     const size_t so = ((size_t)rb * G + g) * 16 + r;

@@ -1,19 +1,31 @@
 // Decode-regime kernel (M <= 16): HBM-bound product of packed b-bit codes with a
 // few activation rows.  Compiled once per bitwidth with -DMATGPTQ_BITS=b.
 // Role of the reference's gptq_matryoshka_simt / gptq_matryoshka at small batch
-// (inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:337-953); the design is its own:
+// (inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:337-953); the design is its own.
 //
-//  * one workgroup owns R row blocks (16 rows each) and all of K; its W waves take
-//    the 128-column tiles of those rows round-robin, so each wave streams whole
-//    tiles with one coalesced 16-byte load per lane and segment;
-//  * codes are turned into exact fp16 integers (c - 2^(b-1)) in registers and fed
-//    to v_mfma_f32_16x16x32_f16 as the 16x32 operand; the activations are the
-//    32x16 operand (columns = batch rows, unused columns are zero), read from an
-//    LDS copy of X when it fits and from global memory otherwise;
-//  * per quantisation group the fp32 tile sum is multiplied by the group scale in
-//    fp32; a general zero point costs one extra MFMA per octet against a constant
-//    operand of ones (sum of x over the group) and no per-weight work;
-//  * the W partial results are combined through LDS and stored as fp16.
+// Work split.  A workgroup has S*W waves and owns S*R row blocks (16 rows each)
+// and all of K.  Wave (s, w) owns the R row blocks of slot s and the 128-column
+// tiles w, w+W, ... of those rows; it streams them with one coalesced 16-byte
+// load per lane and segment, U tiles per pipeline stage.  Two flavours:
+//   stream : the next stage is in flight while the current one is consumed
+//            (two register buffers, fewer waves per SIMD) - long tile runs;
+//   burst  : one register buffer, more waves per SIMD - short tile runs.
+// The W partial sums of a slot meet in LDS at the end.
+//
+// Arithmetic.  The VALU only masks the codes into "raw" fp16 pairs
+// 1024 + c*2^p (one v_and_or_b32 / v_perm_b32 per two codes).  Everything else
+// runs on the matrix cores, with fp32 accumulation, on X' = X * 2^-p staged once
+// per workgroup in LDS (p depends only on the position inside an octet):
+//     D += raw        * X'      ->  sum (1024*2^-p + c) x
+//     D -= (1024 + 2^(b-1) 2^p) * X'   (constant operand)  ->  sum (c - 2^(b-1)) x
+//     D -= (zero-128)/2^(8-b) 2^p * X' (one value per row and group, zero-point form only)
+// so D = sum_k ((c << (8-b)) - zero) x / 2^(8-b) over the group, exact products.
+// Per group the fp32 D is multiplied by the group scale in fp32 and added to
+// the running sum; 2^(8-b) is applied to the final value.
+//
+// Persistence.  When all of X' fits in LDS the grid may be capped: a workgroup then
+// stages X' once and walks several groups of row blocks, with the first loads of the
+// next group in flight while the sums of the current one are combined and stored.
 #include "device_common.h"
 
 #ifndef MATGPTQ_BITS
@@ -26,60 +38,93 @@ namespace {
 
 constexpr int kBits = MATGPTQ_BITS;
 
-// Tiles a wave keeps in flight per pipeline stage, for R row blocks per wave.
+// Tiles a wave loads per pipeline stage, for R row blocks per wave.
 constexpr int tiles_in_flight(int bits, int r) {
   const int u = (16 + r * bits - 1) / (r * bits);
-  return u < 1 ? 1 : (u > 8 ? 8 : u);
+  return u < 1 ? 1 : (u > 4 ? 4 : u);
 }
 
-template <int BITS, int R, int U, bool ZP, bool GROUPED>
-struct Stage {
-  uint32_t w[U][R][BITS];
-  uint2 s[GROUPED ? U : 1][R][GROUPED ? 4 : 1];  // up to 4 groups per tile (g = 32)
-  uint2 z[(GROUPED && ZP) ? U : 1][R][(GROUPED && ZP) ? 4 : 1];
+// fp16 pair constant for pair i of octet J: 2^p in both halves, times `f`.
+template <int BITS, int J, int I>
+__device__ __forceinline__ half2v pow_pair(float f) {
+  return h2_splat(f * (float)(1 << Codec<BITS>::raw_shift(J, I)));
+}
+
+template <int BITS, int J, int I>
+__device__ __forceinline__ half2v inv_pow_pair() {
+  return h2_splat(1.0f / (float)(1 << Codec<BITS>::raw_shift(J, I)));
+}
+
+struct DecodeShape {
+  int S, W;       // slots and k-slices per workgroup
+  int kc;         // tiles of K whose activations are staged in LDS at a time
+  int n_groups;   // groups of S*R row blocks; workgroups walk them with stride gridDim.x
+  int lg_rows;    // log2(S * R * 16)
 };
 
-template <int BITS, int GROUP, bool ZP, int R, bool XLDS>
-__global__ void __launch_bounds__(512)
-decode_kernel(const GemmArgs a) {
+template <int BITS, int R, int U, int GPT, bool ZP>
+struct Stage {
+  uint32_t w[U][R][BITS];
+  uint2 s[U][R][GPT];              // scales of rows 4q..4q+3 (accumulator layout)
+  _Float16 z[ZP ? U : 1][R][GPT];  // zero of row lane%16 (operand layout)
+};
+
+template <int BITS, int GROUP, bool ZP, int R, bool STREAM>
+__device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape sh) {
   constexpr int U = tiles_in_flight(BITS, R);
   constexpr bool GROUPED = GROUP != -1;
   constexpr int GPT = GROUP == 32 ? 4 : 1;  // groups per tile
+  constexpr float kMul = (float)(1 << (8 - BITS));
   extern __shared__ __align__(16) unsigned char smem[];
+  const int S = sh.S, W = sh.W, kc = sh.kc;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int W = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps tile math scalar
+  const int slot = wave / W;
+  const int ws = wave - slot * W;
   const int r16 = lane & 15;  // row of the weight operand / batch column of the x operand
   const int q = lane >> 4;
-  const int rb0 = blockIdx.x * R;
 
-  float* red = reinterpret_cast<float*>(smem);                       // [W][R][256]
-  _Float16* xs = reinterpret_cast<_Float16*>(smem + W * R * 1024);   // [M][K + 8]
-  const int pitch = a.K + 8;
+  // LDS: [ partial sums | X' ]
+  float* red = reinterpret_cast<float*>(smem);                                  // [S*W][R][256]
+  _Float16* xs = reinterpret_cast<_Float16*>(smem + (size_t)S * W * R * 1024);  // [M][kc*128 + 8]
+  const int pitch = kc * 128 + 8;
+  // Operand columns beyond M are never stored, so those lanes simply re-read row M-1.
+  const int xrow = r16 < a.M ? r16 : a.M - 1;
+  const _Float16* xb = xs + xrow * pitch + q * 8;
 
-  const int my_tiles = (a.k_tiles - wave + W - 1) / W;  // tiles wave, wave+W, ...
-  const int n_stages = (my_tiles + U - 1) / U;
+  constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
+  const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
+  const uint32_t aux_bytes = (uint32_t)a.row_blocks * a.G * 32;  // scales / zeros: [N/16][G][16] halves
+  const BufRsrc wres = make_rsrc(a.packed, (uint32_t)a.row_blocks * rb_bytes);
+  const BufRsrc sres = make_rsrc(a.scales, aux_bytes);
+  const BufRsrc zres = make_rsrc(ZP ? a.zeros : a.scales, aux_bytes);
+  const bool single = kc >= a.k_tiles;  // all of X' fits: staged once per workgroup
 
-  const size_t tile_stride = (size_t)tile_words(BITS);
-  const uint32_t* wbase = a.packed + (size_t)rb0 * a.k_tiles * tile_stride;
-  const size_t rb_stride = (size_t)a.k_tiles * tile_stride;
+  using StageT = Stage<BITS, R, U, GPT, ZP>;
+  StageT cur, nxt;
 
-  auto load_stage = [&](Stage<BITS, R, U, ZP, GROUPED>& st, int stage) {
+  // loads stage `stage` of chunk [c0, c1) of the row blocks starting at rb0
+  auto load_stage = [&](StageT& st, int rb0, int c0, int c1, int stage) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
-      const int t = wave + W * (stage * U + u);
-      if (t < a.k_tiles) {
+      const int t = c0 + ws + W * (stage * U + u);
+      if (t < c1) {
 #pragma unroll
         for (int rr = 0; rr < R; rr++) {
-          load_tile_words<BITS>(wbase + rr * rb_stride + (size_t)t * tile_stride, lane, st.w[u][rr]);
+          load_tile_words<BITS>(wres, (uint32_t)(rb0 + rr) * rb_bytes + (uint32_t)t * tile_bytes, lane,
+                                st.w[u][rr]);
           if constexpr (GROUPED) {
 #pragma unroll
             for (int gg = 0; gg < GPT; gg++) {
-              const size_t so = ((size_t)(rb0 + rr) * a.G + (size_t)t * GPT + gg) * 16 + 4 * q;
-              st.s[u][rr][gg] = *reinterpret_cast<const uint2*>(a.scales + so);
-              if constexpr (ZP) st.z[u][rr][gg] = *reinterpret_cast<const uint2*>(a.zeros + so);
+              const uint32_t so = ((uint32_t)(rb0 + rr) * a.G + (uint32_t)t * GPT + gg) * 32;  // bytes
+              const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(sres, q * 8, so, 0);
+              st.s[u][rr][gg] = make_uint2(sv.x, sv.y);
+              if constexpr (ZP) {
+                const uint16_t zv = __builtin_amdgcn_raw_buffer_load_b16(zres, r16 * 2, so, 0);
+                st.z[u][rr][gg] = __builtin_bit_cast(_Float16, zv);
+              }
             }
           }
         }
@@ -87,166 +132,290 @@ decode_kernel(const GemmArgs a) {
     }
   };
 
-  Stage<BITS, R, U, ZP, GROUPED> cur, nxt;
-  if (n_stages > 0) load_stage(cur, 0);
-
-  if constexpr (XLDS) {
-    const int chunks_per_row = a.K >> 3;
-    const int total = a.M * chunks_per_row;
-    for (int i = tid; i < total; i += blockDim.x) {
-      const int m = i / chunks_per_row, c = i - m * chunks_per_row;
-      const uint4 v = reinterpret_cast<const uint4*>(a.x + (size_t)m * a.K)[c];
-      *reinterpret_cast<uint4*>(xs + m * pitch + c * 8) = v;
-    }
-    __syncthreads();
-  }
-
-  float4v acc[R];   // sum over groups of scale * group sum (grouped), unused otherwise
-  float4v d[R];     // running MFMA sum of (c - centre) * x
-  float4v d2;       // running MFMA sum of x (zero-point term)
-#pragma unroll
-  for (int rr = 0; rr < R; rr++) {
-    acc[rr] = float4v{0.f, 0.f, 0.f, 0.f};
-    d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
-  }
-  d2 = float4v{0.f, 0.f, 0.f, 0.f};
-
-  Frag ones;
-  ones.u[0] = ones.u[1] = ones.u[2] = ones.u[3] = 0x3C003C00u;
-
-  constexpr float kMul = (float)(1 << (8 - BITS));
-  constexpr float kInvMul = 1.0f / kMul;
-
-  // acc += scale * (d - (zero - 128) / 2^(8-b) * d2); the common factor 2^(8-b) is applied at the end
-  auto fold_group = [&](const Stage<BITS, R, U, ZP, GROUPED>& st, int u, int gg) {
-#pragma unroll
-    for (int rr = 0; rr < R; rr++) {
-      H4 s;
-      s.v = st.s[u][rr][gg];
-      H4 z;
-      if constexpr (ZP) z.v = st.z[u][rr][gg];
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        float t = d[rr][i];
-        if constexpr (ZP) t -= ((float)z.h[i] - 128.0f) * kInvMul * d2[i];
-        acc[rr][i] += (float)s.h[i] * t;
-        d[rr][i] = 0.f;
+  // X' = X * 2^-p for columns [c0*128, c1*128).  A thread moves eight consecutive k
+  // (one octet of one k-quarter); p depends on the pair inside the octet and, for
+  // b = 2, on the parity of the octet index (k / 32) % 4.
+  auto stage_x = [&](int c0, int c1) {
+    const int chunks = (c1 - c0) * 16;
+    for (int m = 0; m < a.M; m++) {
+      const uint4* src = reinterpret_cast<const uint4*>(a.x + (size_t)m * a.K + (size_t)c0 * 128);
+      for (int c = tid; c < chunks; c += blockDim.x) {
+        Frag v;
+        v.v = src[c];
+        if constexpr (BITS != 8) {
+          const bool odd = BITS == 2 && ((c >> 2) & 1) != 0;  // octet index k/32 = c/4
+          if (odd) {
+            v.p[0] = v.p[0] * inv_pow_pair<BITS, 1, 0>();
+            v.p[1] = v.p[1] * inv_pow_pair<BITS, 1, 1>();
+            v.p[2] = v.p[2] * inv_pow_pair<BITS, 1, 2>();
+            v.p[3] = v.p[3] * inv_pow_pair<BITS, 1, 3>();
+          } else {
+            v.p[0] = v.p[0] * inv_pow_pair<BITS, 0, 0>();
+            v.p[1] = v.p[1] * inv_pow_pair<BITS, 0, 1>();
+            v.p[2] = v.p[2] * inv_pow_pair<BITS, 0, 2>();
+            v.p[3] = v.p[3] * inv_pow_pair<BITS, 0, 3>();
+          }
+        }
+        *reinterpret_cast<uint4*>(xs + m * pitch + c * 8) = v.v;
       }
     }
-    if constexpr (ZP) d2 = float4v{0.f, 0.f, 0.f, 0.f};
   };
 
-  auto octet_step = [&](const Stage<BITS, R, U, ZP, GROUPED>& st, int u, int t, auto jtag) {
+  float4v acc[R];  // sum over groups of scale * D
+  float4v d[R];    // running group sum
+
+  auto fold_group = [&](const uint2 s4, int rr) {
+    H4 s;
+    s.v = s4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[rr][i] += (float)s.h[i] * d[rr][i];
+  };
+
+  auto octet_step = [&](const StageT& st, int u, int tl, auto jtag) {  // tl: tile index inside the LDS copy
     constexpr int J = decltype(jtag)::value;
+#ifdef MATGPTQ_DEBUG_NOCOMPUTE
+    for (int rr = 0; rr < R; rr++) acc[rr][0] += __uint_as_float(st.w[u][rr][J % BITS] & 0x3f000000u);
+    if (tl < 0) acc[0][1] += (float)xb[tl];
+    return;
+#endif
     Frag b;
-    b.v = make_uint4(0u, 0u, 0u, 0u);
-    if (r16 < a.M) {
-      const int kk = t * 128 + J * 32 + q * 8;
-      if constexpr (XLDS)
-        b.v = *reinterpret_cast<const uint4*>(xs + r16 * pitch + kk);
-      else
-        b.v = *reinterpret_cast<const uint4*>(a.x + (size_t)r16 * a.K + kk);
-    }
+    b.v = *reinterpret_cast<const uint4*>(xb + tl * 128 + J * 32);
+    // constant operand  -(1024 + centre * 2^p)
+    Frag bias;
+    constexpr float cc = (float)Codec<BITS>::kCentre;
+    bias.p[0] = h2_splat(-1024.0f) - pow_pair<BITS, J, 0>(cc);
+    bias.p[1] = h2_splat(-1024.0f) - pow_pair<BITS, J, 1>(cc);
+    bias.p[2] = h2_splat(-1024.0f) - pow_pair<BITS, J, 2>(cc);
+    bias.p[3] = h2_splat(-1024.0f) - pow_pair<BITS, J, 3>(cc);
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
       Frag aw;
-      centred_octet<BITS, J>(st.w[u][rr], aw);
-      d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw.h, b.h, d[rr], 0, 0, 0);
+      raw_octet<BITS, J>(st.w[u][rr], aw.u);
+      // a group's first product starts from a zero accumulator operand
+      constexpr bool kFresh = GROUP == 32 || (GROUP == 128 && J == 0);
+      const float4v zero4 = {0.f, 0.f, 0.f, 0.f};
+      d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw.h, b.h, kFresh ? zero4 : d[rr], 0, 0, 0);
+      d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bias.h, b.h, d[rr], 0, 0, 0);
+      if constexpr (ZP) {
+        // -(zero - 128) / 2^(8-b) * 2^p for this lane's row: exact in fp16
+        _Float16 zv;
+        if constexpr (GROUPED) zv = st.z[u][rr][GROUP == 32 ? J : 0];
+        else zv = st.z[0][rr][0];
+        const _Float16 zrel = (_Float16)128.0f - zv;
+        const half2v z2 = {zrel, zrel};
+        Frag az;
+        az.p[0] = z2 * pow_pair<BITS, J, 0>(1.0f / kMul);
+        az.p[1] = z2 * pow_pair<BITS, J, 1>(1.0f / kMul);
+        az.p[2] = z2 * pow_pair<BITS, J, 2>(1.0f / kMul);
+        az.p[3] = z2 * pow_pair<BITS, J, 3>(1.0f / kMul);
+        d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(az.h, b.h, d[rr], 0, 0, 0);
+      }
+      if constexpr (GROUP == 32) fold_group(st.s[u][rr][J], rr);
     }
-    if constexpr (ZP) d2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones.h, b.h, d2, 0, 0, 0);
-    if constexpr (GROUP == 32) fold_group(st, u, J);
   };
 
-  for (int stage = 0; stage < n_stages; stage++) {
-    if (stage + 1 < n_stages) load_stage(nxt, stage + 1);
+  auto compute_stage = [&](const StageT& st, int c0, int c1, int stage) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
-      const int t = wave + W * (stage * U + u);
-      if (t < a.k_tiles) {
-        octet_step(cur, u, t, std::integral_constant<int, 0>{});
-        octet_step(cur, u, t, std::integral_constant<int, 1>{});
-        octet_step(cur, u, t, std::integral_constant<int, 2>{});
-        octet_step(cur, u, t, std::integral_constant<int, 3>{});
-        if constexpr (GROUP == 128) fold_group(cur, u, 0);
+      const int t = c0 + ws + W * (stage * U + u);
+      if (t < c1) {
+        const int tl = t - c0;
+        octet_step(st, u, tl, std::integral_constant<int, 0>{});
+        octet_step(st, u, tl, std::integral_constant<int, 1>{});
+        octet_step(st, u, tl, std::integral_constant<int, 2>{});
+        octet_step(st, u, tl, std::integral_constant<int, 3>{});
+        if constexpr (GROUP == 128) {
+#pragma unroll
+          for (int rr = 0; rr < R; rr++) fold_group(st.s[u][rr][0], rr);
+        }
       }
     }
-    if (stage + 1 < n_stages) cur = nxt;
+  };
+
+  auto stages_of = [&](int c0, int c1, bool live) {
+    const int span = c1 - c0 - ws;  // this wave owns tiles c0+ws, c0+ws+W, ... below c1
+    const int my_tiles = (live && span > 0) ? (span + W - 1) / W : 0;
+    return (my_tiles + U - 1) / U;
+  };
+
+  int it = blockIdx.x;
+  bool have_first = false;  // stage 0 of the coming group is already in `cur`
+  if (single) {
+    const int rb0 = (it * S + slot) * R;
+    if (it < sh.n_groups && rb0 < a.row_blocks && ws < a.k_tiles) {
+      load_stage(cur, rb0, 0, a.k_tiles, 0);  // weights first: they have the longest way to come
+      have_first = true;
+    }
+#ifndef MATGPTQ_DEBUG_NOSTAGE
+    stage_x(0, a.k_tiles);
+    __syncthreads();
+#endif
   }
 
-  if constexpr (!GROUPED) {
-    // one scale (and zero) per row: fold once
+  for (; it < sh.n_groups; it += gridDim.x) {
+    const int rb_wg = it * S * R;          // first row block of the group
+    const int rb0 = rb_wg + slot * R;      // first row block of this wave
+    const bool live = rb0 < a.row_blocks;  // the last group may have idle slots
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
-      const size_t so = (size_t)(rb0 + rr) * 16 + 4 * q;
-      H4 s, z;
-      s.v = *reinterpret_cast<const uint2*>(a.scales + so);
-      if constexpr (ZP) z.v = *reinterpret_cast<const uint2*>(a.zeros + so);
+      acc[rr] = float4v{0.f, 0.f, 0.f, 0.f};
+      d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
+    }
+    if constexpr (!GROUPED && ZP) {
+      if (live) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        float t = d[rr][i];
-        if constexpr (ZP) t -= ((float)z.h[i] - 128.0f) * kInvMul * d2[i];
-        acc[rr][i] = (float)s.h[i] * t;
+        for (int rr = 0; rr < R; rr++)
+        {
+          const _Float16 zv = reinterpret_cast<const _Float16*>(a.zeros)[(size_t)(rb0 + rr) * 16 + r16];
+          cur.z[0][rr][0] = zv;
+          if constexpr (STREAM) nxt.z[0][rr][0] = zv;
+        }
       }
     }
-  }
 
-  // combine the W partial sums: red[wave][rr][lane*4 + i]
+    // K is walked in chunks of kc tiles so that the LDS copy of X' stays small.
+    for (int c0 = 0; c0 < a.k_tiles; c0 += kc) {
+      const int c1 = c0 + kc < a.k_tiles ? c0 + kc : a.k_tiles;
+      const int n_stages = stages_of(c0, c1, live);
+      if (!have_first && n_stages > 0) load_stage(cur, rb0, c0, c1, 0);
+      have_first = false;
+      if (!single) {
+        __syncthreads();  // all waves are done with the previous contents of X'
+        stage_x(c0, c1);
+        __syncthreads();
+      }
+
+      // next group's first stage, issued as soon as a register buffer is free
+      const int it_next = it + (int)gridDim.x;
+      auto prefetch_next = [&]() {
+        if (single && it_next < sh.n_groups) {
+          const int rbn = (it_next * S + slot) * R;
+          if (rbn < a.row_blocks && ws < a.k_tiles) {
+            load_stage(cur, rbn, 0, a.k_tiles, 0);
+            have_first = true;
+          }
+        }
+      };
+
+      if constexpr (STREAM) {
+        // two stages per trip so that the prefetched stage needs no register copy
+        for (int stage = 0; stage < n_stages; stage += 2) {
+          if (stage + 1 < n_stages) load_stage(nxt, rb0, c0, c1, stage + 1);
+          compute_stage(cur, c0, c1, stage);
+          if (stage + 1 < n_stages) {
+            if (stage + 2 < n_stages) load_stage(cur, rb0, c0, c1, stage + 2);
+            else prefetch_next();
+            compute_stage(nxt, c0, c1, stage + 1);
+          } else {
+            prefetch_next();
+          }
+        }
+        if (n_stages == 0) prefetch_next();
+      } else {
+        for (int stage = 0; stage < n_stages; stage++) {
+          if (stage > 0) load_stage(cur, rb0, c0, c1, stage);
+          compute_stage(cur, c0, c1, stage);
+        }
+        prefetch_next();
+      }
+    }
+
+    if constexpr (!GROUPED) {
+      if (live) {
 #pragma unroll
-  for (int rr = 0; rr < R; rr++)
-    *reinterpret_cast<float4v*>(red + ((wave * R + rr) * 64 + lane) * 4) = acc[rr];
-  __syncthreads();
+        for (int rr = 0; rr < R; rr++)
+          fold_group(*reinterpret_cast<const uint2*>(a.scales + (size_t)(rb0 + rr) * 16 + 4 * q), rr);
+      }
+    }
 
-  const int outs = R * 16 * a.M;
-  for (int o = tid; o < outs; o += blockDim.x) {
-    const int n = o / (R * 16);
-    const int rowl = o - n * (R * 16);
-    const int rr = rowl >> 4, row = rowl & 15;
-    const int idx = (((row >> 2) * 16 + n) << 2) + (row & 3);
-    float sum = 0.f;
-    for (int w = 0; w < W; w++) sum += red[(w * R + rr) * 256 + idx];
-    const _Float16 h = (_Float16)(sum * kMul);
-    reinterpret_cast<_Float16*>(a.y)[(size_t)n * a.N + (size_t)(rb0 + rr) * 16 + row] = h;
+#ifdef MATGPTQ_DEBUG_NOREDUCE
+    if (acc[0][0] == 1.2345f) a.y[tid] = 1;
+    continue;
+#endif
+    // combine the W partial sums of each slot: red[wave][rr][lane*4 + i]
+    if (it != (int)blockIdx.x) __syncthreads();  // the previous group's sums have been read
+#pragma unroll
+    for (int rr = 0; rr < R; rr++)
+      *reinterpret_cast<float4v*>(red + ((wave * R + rr) * 64 + lane) * 4) = acc[rr];
+    __syncthreads();
+
+    const int outs = a.M << sh.lg_rows;
+    for (int o = tid; o < outs; o += blockDim.x) {
+      const int n = o >> sh.lg_rows;
+      const int rowl = o & ((1 << sh.lg_rows) - 1);
+      const int rbl = rowl >> 4, row = rowl & 15;  // row block inside the group
+      const int sl = rbl / R, rr = rbl % R;
+      const int grow = (rb_wg + rbl) * 16 + row;
+      if (grow < a.N) {
+        const float* src = red + ((sl * W) * R + rr) * 256 + (((row >> 2) * 16 + n) << 2) + (row & 3);
+        float sum = 0.f;
+        for (int w = 0; w < W; w++) sum += src[w * R * 256];
+        reinterpret_cast<_Float16*>(a.y)[(size_t)n * a.N + grow] = (_Float16)(sum * kMul);
+      }
+    }
   }
 }
 
-template <int GROUP, bool ZP, int R, bool XLDS>
-hipError_t launch_one(const GemmArgs& a, int W, size_t smem, hipStream_t stream) {
-  const dim3 grid(a.row_blocks / R), block(64 * W);
-  hipLaunchKernelGGL((decode_kernel<kBits, GROUP, ZP, R, XLDS>), grid, block, smem, stream, a);
+// stream: up to 16 waves per workgroup, 128 VGPRs
+template <int BITS, int GROUP, bool ZP, int R>
+__global__ void __launch_bounds__(1024)
+decode_stream_kernel(const GemmArgs a, const DecodeShape sh) {
+  decode_body<BITS, GROUP, ZP, R, true>(a, sh);
+}
+
+// burst: up to 8 waves per workgroup, register budget for 6 waves per SIMD
+template <int BITS, int GROUP, bool ZP, int R>
+__global__ void __launch_bounds__(512, 6)
+decode_burst_kernel(const GemmArgs a, const DecodeShape sh) {
+  decode_body<BITS, GROUP, ZP, R, false>(a, sh);
+}
+
+template <int GROUP, bool ZP, int R>
+hipError_t launch_one(const GemmArgs& a, int S, int W, int kc, int max_wgs, bool stream_flavour,
+                      size_t smem, hipStream_t stream) {
+  const int per_wg = S * R;
+  const int n_groups = (a.row_blocks + per_wg - 1) / per_wg;
+  int lg = 4;
+  while ((1 << lg) < per_wg * 16) lg++;
+  const dim3 grid(max_wgs > 0 && max_wgs < n_groups ? max_wgs : n_groups), block(64 * S * W);
+  const DecodeShape sh{S, W, kc, n_groups, lg};
+  if (stream_flavour)
+    hipLaunchKernelGGL((decode_stream_kernel<kBits, GROUP, ZP, R>), grid, block, smem, stream, a, sh);
+  else
+    hipLaunchKernelGGL((decode_burst_kernel<kBits, GROUP, ZP, R>), grid, block, smem, stream, a, sh);
   return hipGetLastError();
 }
 
 template <int GROUP, bool ZP>
-hipError_t launch_rx(const GemmArgs& a, int R, int W, bool xlds, size_t smem, hipStream_t s) {
-  if (xlds) {
-    if (R == 1) return launch_one<GROUP, ZP, 1, true>(a, W, smem, s);
-    if (R == 2) return launch_one<GROUP, ZP, 2, true>(a, W, smem, s);
-    return launch_one<GROUP, ZP, 4, true>(a, W, smem, s);
-  }
-  if (R == 1) return launch_one<GROUP, ZP, 1, false>(a, W, smem, s);
-  if (R == 2) return launch_one<GROUP, ZP, 2, false>(a, W, smem, s);
-  return launch_one<GROUP, ZP, 4, false>(a, W, smem, s);
+hipError_t launch_r(const GemmArgs& a, int R, int S, int W, int kc, int max_wgs, bool sf,
+                    size_t smem, hipStream_t s) {
+  if (R == 1) return launch_one<GROUP, ZP, 1>(a, S, W, kc, max_wgs, sf, smem, s);
+  if (R == 2) return launch_one<GROUP, ZP, 2>(a, S, W, kc, max_wgs, sf, smem, s);
+  return launch_one<GROUP, ZP, 4>(a, S, W, kc, max_wgs, sf, smem, s);
 }
 
 }  // namespace
 
 // Entry of this translation unit: launch the decode kernel for bitwidth MATGPTQ_BITS.
-// R in {1,2,4} row blocks per workgroup, W in {1..8} waves, xlds: stage X in LDS.
+// R in {1,2,4} row blocks per wave, S slots and W k-slices per workgroup
+// (S*W <= 16 for the stream flavour, <= 8 for burst), kc = tiles of K staged in LDS at
+// a time, max_wgs = cap on the grid (0 = one workgroup per group of row blocks; otherwise
+// workgroups walk several groups), smem = dynamic LDS bytes (see decode_lds_bytes in abi.hip).
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
-hipError_t MATGPTQ_CAT(launch_decode_b, MATGPTQ_BITS)(const GemmArgs& a, int group_size,
-                                                      int R, int W, bool xlds,
+hipError_t MATGPTQ_CAT(launch_decode_b, MATGPTQ_BITS)(const GemmArgs& a, int group_size, int R,
+                                                      int S, int W, int kc, int max_wgs,
+                                                      bool stream_flavour, size_t smem,
                                                       hipStream_t stream) {
   const bool zp = a.zeros != nullptr;
-  const size_t smem = (size_t)W * R * 1024 + (xlds ? (size_t)a.M * (a.K + 8) * 2 : 0);
   if (group_size == 128)
-    return zp ? launch_rx<128, true>(a, R, W, xlds, smem, stream)
-              : launch_rx<128, false>(a, R, W, xlds, smem, stream);
+    return zp ? launch_r<128, true>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream)
+              : launch_r<128, false>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream);
   if (group_size == 32)
-    return zp ? launch_rx<32, true>(a, R, W, xlds, smem, stream)
-              : launch_rx<32, false>(a, R, W, xlds, smem, stream);
-  return zp ? launch_rx<-1, true>(a, R, W, xlds, smem, stream)
-            : launch_rx<-1, false>(a, R, W, xlds, smem, stream);
+    return zp ? launch_r<32, true>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream)
+              : launch_r<32, false>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream);
+  return zp ? launch_r<-1, true>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream)
+            : launch_r<-1, false>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream);
 }
 
 }  // namespace matgptq

@@ -55,11 +55,72 @@ __device__ __forceinline__ half2v centre_raw(uint32_t raw, int centre) {
   }
 }
 
+// (x & mask) | orv in one VALU instruction.  `mask` travels in an SGPR and `orv`
+// in a VGPR: a VOP3 encoding of this target takes no literal and one scalar operand.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t orv) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(orv));
+  return r;
+}
+
+// Device form of Codec<BITS>::decode_octet (same results, fewer instructions):
+// the four raw pairs 1024 + c * 2^p of octet J.
+template <int BITS, int J>
+__device__ __forceinline__ void raw_octet(const uint32_t (&w)[BITS], uint32_t (&r)[4]) {
+  const uint32_t magic = kMagic;
+  if constexpr (BITS == 4 || BITS == 3) {
+    uint32_t x;
+    if constexpr (BITS == 4) {
+      x = w[J];
+    } else {
+      const uint32_t lo = (w[J >> 1] >> (2 * (J & 1))) & 0x33333333u;
+      const uint32_t c = w[2];
+      const uint32_t cs = J == 0 ? (c << 2) : J == 1 ? (c << 1) : J == 2 ? c : (c >> 1);
+      x = and_or(cs, 0x44444444u, lo);
+    }
+    const uint32_t x8 = x >> 8;
+    r[0] = and_or(x, 0x000F000Fu, magic);
+    r[1] = and_or(x, 0x00F000F0u, magic);
+    r[2] = and_or(x8, 0x000F000Fu, magic);
+    r[3] = and_or(x8, 0x00F000F0u, magic);
+  } else if constexpr (BITS == 2) {
+    const uint32_t x = w[J >> 1];
+    const uint32_t x6 = x >> 6;
+    if constexpr ((J & 1) == 0) {
+      r[0] = and_or(x, 0x00030003u, magic);
+      r[1] = and_or(x, 0x000C000Cu, magic);
+      r[2] = and_or(x, 0x00300030u, magic);
+      r[3] = and_or(x6, 0x00030003u, magic);
+    } else {
+      const uint32_t x12 = x >> 12;
+      r[0] = and_or(x6, 0x000C000Cu, magic);
+      r[1] = and_or(x6, 0x00300030u, magic);
+      r[2] = and_or(x12, 0x00030003u, magic);
+      r[3] = and_or(x12, 0x000C000Cu, magic);
+    }
+  } else if constexpr (BITS == 6) {
+    const uint32_t h = w[J], h8 = h >> 8;
+    const uint32_t l = (J & 1) ? (w[4 + (J >> 1)] >> 8) : w[4 + (J >> 1)];
+    const uint32_t l2 = l >> 2;
+    r[0] = ((h & 0x000F000Fu) << 2) | and_or(l, 0x00030003u, magic);
+    r[1] = ((h & 0x00F000F0u) << 2) | and_or(l, 0x00300030u, magic);
+    r[2] = ((h8 & 0x000F000Fu) << 2) | and_or(l2, 0x00030003u, magic);
+    r[3] = ((h8 & 0x00F000F0u) << 2) | and_or(l2, 0x00300030u, magic);
+  } else {
+    // bytes: pair 2d = (byte0, byte2) of word 2J+d, pair 2d+1 = (byte1, byte3)
+    const uint32_t fill = 0x64646464u;
+    r[0] = __builtin_amdgcn_perm(fill, w[2 * J], 0x04020400u);
+    r[1] = __builtin_amdgcn_perm(fill, w[2 * J], 0x04030401u);
+    r[2] = __builtin_amdgcn_perm(fill, w[2 * J + 1], 0x04020400u);
+    r[3] = __builtin_amdgcn_perm(fill, w[2 * J + 1], 0x04030401u);
+  }
+}
+
 // Octet j of a lane -> MFMA operand holding (c - 2^(b-1)) for its eight codes.
 template <int BITS, int J>
 __device__ __forceinline__ void centred_octet(const uint32_t (&w)[BITS], Frag& a) {
   uint32_t raw[4];
-  Codec<BITS>::decode_octet(w, J, raw);
+  raw_octet<BITS, J>(w, raw);
   constexpr int c = Codec<BITS>::kCentre;
   a.p[0] = centre_raw<Codec<BITS>::raw_shift(J, 0)>(raw[0], c);
   a.p[1] = centre_raw<Codec<BITS>::raw_shift(J, 1)>(raw[1], c);
@@ -67,7 +128,49 @@ __device__ __forceinline__ void centred_octet(const uint32_t (&w)[BITS], Frag& a
   a.p[3] = centre_raw<Codec<BITS>::raw_shift(J, 3)>(raw[3], c);
 }
 
-// Loads the BITS words of `lane` from a tile with one load per segment.
+// Buffer resources: a 128-bit scalar descriptor (base, byte size) lets every load
+// take its wave-uniform part from an SGPR and its per-lane part from one 32-bit
+// VGPR, so a stream of tile loads needs no vector address arithmetic; reads past
+// the size return zero.  Offsets are 32-bit: a tensor must stay below 4 GiB.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __amdgpu_buffer_rsrc_t BufRsrc;
+constexpr int kAuxStream = 2;  // "nt": data that is read once
+
+__device__ __forceinline__ BufRsrc make_rsrc(const void* p, uint32_t bytes) {
+  // word 3 = 0x00020000: untyped 32-bit data format of this target's buffer descriptors
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+// Loads the BITS words of `lane` from the tile that starts `tile_bytes` into the buffer
+// (wave-uniform), one load per segment, as streaming reads.
+template <int BITS>
+__device__ __forceinline__ void load_tile_words(BufRsrc rs, uint32_t tile_bytes, int lane,
+                                                uint32_t (&w)[BITS]) {
+  if constexpr (BITS == 2) {
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, tile_bytes, kAuxStream);
+    w[0] = v.x; w[1] = v.y;
+  } else if constexpr (BITS == 3) {
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, tile_bytes, kAuxStream);
+    w[0] = v.x; w[1] = v.y;
+    w[2] = __builtin_amdgcn_raw_buffer_load_b32(rs, 512 + lane * 4, tile_bytes, kAuxStream);
+  } else if constexpr (BITS == 4) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, tile_bytes, kAuxStream);
+    w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+  } else if constexpr (BITS == 6) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, tile_bytes, kAuxStream);
+    w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    const u32x2 l = __builtin_amdgcn_raw_buffer_load_b64(rs, 1024 + lane * 8, tile_bytes, kAuxStream);
+    w[4] = l.x; w[5] = l.y;
+  } else {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rs, lane * 16, tile_bytes, kAuxStream);
+    w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    const u32x4 l = __builtin_amdgcn_raw_buffer_load_b128(rs, 1024 + lane * 16, tile_bytes, kAuxStream);
+    w[4] = l.x; w[5] = l.y; w[6] = l.z; w[7] = l.w;
+  }
+}
+
+// Same from a plain pointer (load-time kernels).
 template <int BITS>
 __device__ __forceinline__ void load_tile_words(const uint32_t* __restrict__ tile, int lane,
                                                 uint32_t (&w)[BITS]) {

@@ -106,29 +106,31 @@ struct Codec<4> {
 
 // ----- b = 2 --------------------------------------------------------------
 // Word d holds octets 2d and 2d+1 as sixteen 2-bit fields.  In each 16-bit half
-// field i (bits 2i, 2i+1) belongs to pair i: pairs 0..3 are octet 2d, pairs
+// field f (bits 2f, 2f+1) belongs to pair f: pairs 0..3 are octet 2d, pairs
 // 4..7 octet 2d+1; the low half holds the even element, the high half the odd.
-// Fields 0..4 are read in place (p = 2i), fields 5..7 after a shift by 10.
+// Fields 0..2 are read in place, 3..5 after a shift by 6, 6..7 after a shift by
+// 12, so that no field sits higher than bit 4 of the mantissa (p <= 4).
 template <>
 struct Codec<2> {
   static constexpr int kCentre = 2;
   static constexpr int raw_shift(int j, int i) {
     const int f = (j & 1) * 4 + i;  // field index in the half word
-    return f < 5 ? 2 * f : 2 * (f - 5);
+    return 2 * (f % 3);
   }
   MATGPTQ_HD static void decode_octet(const uint32_t (&w)[2], int j, uint32_t (&r)[4]) {
     const uint32_t x = w[j >> 1];
+    const uint32_t x6 = x >> 6;
     if ((j & 1) == 0) {
       r[0] = (x & 0x00030003u) | kMagic;
       r[1] = (x & 0x000C000Cu) | kMagic;
       r[2] = (x & 0x00300030u) | kMagic;
-      r[3] = (x & 0x00C000C0u) | kMagic;
+      r[3] = (x6 & 0x00030003u) | kMagic;
     } else {
-      const uint32_t x10 = x >> 10;
-      r[0] = (x & 0x03000300u) | kMagic;
-      r[1] = (x10 & 0x00030003u) | kMagic;
-      r[2] = (x10 & 0x000C000Cu) | kMagic;
-      r[3] = (x10 & 0x00300030u) | kMagic;
+      const uint32_t x12 = x >> 12;
+      r[0] = (x6 & 0x000C000Cu) | kMagic;
+      r[1] = (x6 & 0x00300030u) | kMagic;
+      r[2] = (x12 & 0x00030003u) | kMagic;
+      r[3] = (x12 & 0x000C000Cu) | kMagic;
     }
   }
   MATGPTQ_HD static void encode_lane(const uint8_t (&codes)[32], uint32_t (&w)[2]) {

@@ -51,7 +51,7 @@ template <int BITS, int J, bool ZP>
 __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], half2v zrel, half2v scale,
                                               Frag& a) {
   uint32_t raw[4];
-  Codec<BITS>::decode_octet(w, J, raw);
+  raw_octet<BITS, J>(w, raw);
   a.p[0] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 0), ZP>(raw[0], zrel, scale);
   a.p[1] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 1), ZP>(raw[1], zrel, scale);
   a.p[2] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 2), ZP>(raw[2], zrel, scale);
@@ -82,8 +82,9 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   const int m0 = mtile * TM;
   const int rb_first = (nt * 4 + wave) * RBW;
 
-  const size_t tile_stride = (size_t)tile_words(BITS);
-  const size_t rb_stride = (size_t)a.k_tiles * tile_stride;
+  constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
+  const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
+  const BufRsrc wres = make_rsrc(a.packed, (uint32_t)a.row_blocks * rb_bytes);
 
   float4v acc[RBW][MT];
 #pragma unroll
@@ -101,7 +102,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     for (int rr = 0; rr < RBW; rr++) {
       const int rb = rb_first + rr;
       if (rb < a.row_blocks) {
-        load_tile_words<BITS>(a.packed + rb * rb_stride + (size_t)kb * tile_stride, lane, w[rr]);
+        load_tile_words<BITS>(wres, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
 #pragma unroll
         for (int gg = 0; gg < GPT; gg++) {
           const size_t g = GROUP == -1 ? 0 : (size_t)kb * GPT + gg;

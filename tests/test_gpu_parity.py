@@ -1,0 +1,215 @@
+"""HIP path against the oracle, through the C ABI, on a real MI355X.
+
+Integer results (slice, pack, unpack) and the dense dequantised weight must be
+bit-exact; GEMM outputs must be within the tolerance stated in tests/_gpu_util.py.
+"""
+import numpy as np
+import pytest
+import torch
+
+from matgptq_amd import _lib
+from oracle import matgptq_oracle as o
+from tests import _gpu_util as G
+
+pytestmark = pytest.mark.gpu
+BITS = (2, 3, 4, 6, 8)
+GROUPS = (128, 32, -1)
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_slice_pack_unpack_bit_exact(b):
+    L = G.lib()
+    rng = np.random.default_rng(b)
+    n, k = 80, 640
+    q = rng.integers(0, 256, (n, k), dtype=np.uint8)
+    q[0, :256] = np.arange(256, dtype=np.uint8)  # every master code appears
+    ref = o.slice_codes(q, b)
+    qd = G.to_dev(q)
+    sl = torch.empty_like(qd)
+    _lib.check(L.matgptq_slice_device(qd.data_ptr(), q.size, b, sl.data_ptr(), G.stream()))
+    assert np.array_equal(sl.cpu().numpy(), ref)
+    # device pack (slicing in registers) == host pack, word for word
+    host = np.zeros(L.matgptq_packed_words(b, n, k), dtype=np.uint32)
+    _lib.check(L.matgptq_pack_host(q.ctypes.data, n, k, b, 1, host.ctypes.data))
+    dev = G.pack_device(q, b, from_master=True)
+    assert np.array_equal(dev.cpu().numpy().view(np.uint32), host)
+    assert np.array_equal(G.pack_device(ref, b, from_master=False).cpu().numpy().view(np.uint32), host)
+    # the codes the GEMM kernels see (device unpack uses their unpack sequence)
+    back = torch.empty(n, k, dtype=torch.uint8, device=G.DEV)
+    _lib.check(L.matgptq_unpack_device(dev.data_ptr(), n, k, b, back.data_ptr(), G.stream()))
+    assert np.array_equal(back.cpu().numpy(), ref)
+
+
+def test_slice_device_odd_length():
+    L = G.lib()
+    q = np.arange(1003, dtype=np.int64).astype(np.uint8)
+    qd = G.to_dev(q)
+    out = torch.zeros_like(qd)
+    _lib.check(L.matgptq_slice_device(qd.data_ptr(), q.size, 3, out.data_ptr(), G.stream()))
+    assert np.array_equal(out.cpu().numpy(), o.slice_codes(q, 3))
+    _lib.check(L.matgptq_slice_device(None, 0, 3, None, G.stream()))  # empty input is a no-op
+
+
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_dequantize_bit_exact(b, g, golden):
+    L = G.lib()
+    lay = G.Layer(48, 512, b, g, seed=10 + b)
+    w = torch.empty(48, 512, dtype=torch.float16, device=G.DEV)
+    _lib.check(L.matgptq_dequantize_device(b, g, 48, 512, lay.packed.data_ptr(), lay.scales.data_ptr(),
+                                           lay.zeros.data_ptr(), w.data_ptr(), G.stream()))
+    assert np.array_equal(w.cpu().numpy().view(np.uint16), lay.w.view(np.uint16))
+    if g == 128:  # and against the vectors the reference's own dequantize produced
+        n, k = golden["q"].shape
+        pk = G.pack_device(golden["q"], b, True)
+        sd, zd = G.reorder_device(golden["scale"], n, k, g), G.reorder_device(golden["zero"], n, k, g)
+        w = torch.empty(n, k, dtype=torch.float16, device=G.DEV)
+        _lib.check(L.matgptq_dequantize_device(b, g, n, k, pk.data_ptr(), sd.data_ptr(), zd.data_ptr(),
+                                               w.data_ptr(), G.stream()))
+        assert np.array_equal(w.cpu().numpy().view(np.uint16), golden[f"w_b{b}"].view(np.uint16))
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_forward_against_reference_vectors(b, golden):
+    # FakeMatryoshkaLinear.forward of the reference on its own small layer (M = 3 -> decode path)
+    n, k = golden["q"].shape
+    pk = G.pack_device(golden["q"], b, True)
+    sd, zd = G.reorder_device(golden["scale"], n, k, 128), G.reorder_device(golden["zero"], n, k, 128)
+    y = G.gemm(b, 128, n, k, G.to_dev(golden["x"]), pk, sd, zd).cpu().numpy()
+    ref = golden[f"y_b{b}"].astype(np.float64)
+    assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+    G.assert_close_to_oracle(y, golden["x"], golden[f"w_b{b}"], f"golden b={b}")
+
+
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_decode_parity(b, g, zp):
+    lay = G.Layer(64, 1024, b, g, seed=b, zero_points=zp)
+    for m in (1, 2, 3, 5, 8, 16):
+        x = o.make_activations(m, 1024, seed=m)
+        G.assert_close_to_oracle(lay.run(x), x, lay.w, f"decode b={b} g={g} zp={zp} M={m}")
+
+
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_prefill_parity(b, g, zp):
+    lay = G.Layer(336, 512, b, g, seed=20 + b, zero_points=zp)  # 21 row blocks: ragged workgroups
+    for m in (17, 64, 100, 257):
+        x = o.make_activations(m, 512, seed=m)
+        G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
+
+
+@pytest.mark.parametrize("cfg", range(5))
+def test_prefill_every_tile_configuration(cfg):
+    lay = G.Layer(1040, 1024, 4, 128, seed=3)
+    x = o.make_activations(300, 1024, seed=1)
+    G.assert_close_to_oracle(lay.run(x, flags=1 | ((64 + cfg) << 8)), x, lay.w, f"cfg {cfg}")
+
+
+def _decode_variants():
+    out = []
+    for v in range(1, 43):
+        for flavour in (1, 2):
+            for cap in (1, 2):
+                out.append(1 | (v << 8) | (flavour << 16) | (cap << 18))
+    return out
+
+
+def test_decode_every_work_split():
+    # all (R, S, W) shapes, both flavours, capped (persistent) and uncapped grids; 65 row
+    # blocks leave idle slots in the last group, K = 4096 gives up to 32 tiles per wave
+    lay = G.Layer(1040, 4096, 4, 128, seed=4)
+    x = o.make_activations(3, 4096, seed=2)
+    ran = 0
+    for flags in _decode_variants():
+        try:
+            y = lay.run(x, flags=flags)
+        except _lib.MatGPTQError as e:
+            assert "variant" in str(e)
+            continue
+        G.assert_close_to_oracle(y, x, lay.w, f"flags {flags:#x}")
+        ran += 1
+    assert ran >= 100
+
+
+@pytest.mark.parametrize("b", (3, 4))
+@pytest.mark.parametrize("m", (2, 4, 8, 16))
+def test_small_batch_with_outlier_channels(b, m):
+    # 1 % of the channels scaled by 20: stresses the fp32 accumulation
+    lay = G.Layer(256, 4096, b, 128, seed=30 + m)
+    x = o.make_activations(m, 4096, seed=m, outlier_frac=0.01, outlier_gain=20.0)
+    G.assert_close_to_oracle(lay.run(x), x, lay.w, f"outliers b={b} M={m}")
+
+
+def test_chunked_activation_staging():
+    # M = 16 with K = 14336 does not fit in LDS at once: the kernel walks K in chunks
+    lay = G.Layer(64, 14336, 4, 128, seed=7)
+    x = o.make_activations(16, 14336, seed=7)
+    assert "kc112" not in _lib.describe_plan(4, 128, 64, 14336, 16, True)
+    G.assert_close_to_oracle(lay.run(x), x, lay.w, "chunked")
+
+
+@pytest.mark.parametrize("gsz", (-1, 32, 128))
+@pytest.mark.parametrize("m", (1, 8, 16))
+@pytest.mark.parametrize("k", (1024, 4096, 8192))
+@pytest.mark.parametrize("b", BITS)
+def test_reference_kernel_test_grid(b, k, m, gsz):
+    # the reference's own test (inference_lib/test_matgptq_matmul.py:11-49), fp16 half of
+    # it: codes < 2^b, scales in {0,1}, integer activations, N = 16, symmetric form.
+    # All arithmetic is exact, so the result must equal the closed form bit for bit.
+    rng = np.random.default_rng(1)
+    n = 16
+    g = k if gsz == -1 else gsz
+    codes = rng.integers(0, 1 << b, (n, k), dtype=np.uint8)
+    scales = np.round(rng.random((n, k // g))).astype(np.float16)
+    x = np.round(rng.standard_normal((m, k))).astype(np.float16)
+    w = o.dequantize_kernel_form(codes, scales, b, gsz)
+    expect = o.linear_f64(x, w).astype(np.float16)
+    pk = G.pack_device(codes, b, from_master=False)
+    sd = G.reorder_device(scales, n, k, gsz)
+    y = G.gemm(b, gsz, n, k, G.to_dev(x), pk, sd, None).cpu().numpy()
+    assert np.array_equal(y.view(np.uint16), expect.view(np.uint16))
+
+
+LLAMA8B = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "down": (4096, 14336)}
+
+
+@pytest.mark.parametrize("name", sorted(LLAMA8B))
+@pytest.mark.parametrize("b", BITS)
+def test_llama3_8b_layers_decode_full_size(name, b):
+    n, k = LLAMA8B[name]
+    lay = G.Layer(n, k, b, 128, seed=0)
+    x = o.make_activations(1, k, seed=0)
+    y = lay.run(x)
+    G.assert_close_to_oracle(y, x, lay.w, f"{name} b={b}")
+    # linearity in x at full size: f(2x) = 2 f(x) up to the last bit of the fp16 result
+    # (activations are pre-scaled by powers of two inside the kernel, so the smallest of
+    # them may round differently after doubling)
+    y2 = lay.run((x.astype(np.float32) * 2).astype(np.float16)).astype(np.float64)
+    assert np.max(np.abs(y2 - 2.0 * y.astype(np.float64))) <= 2.0 ** -9 * np.max(np.abs(y2))
+
+
+def test_llama3_70b_layer_prefill_full_size():
+    n, k, m = 8192, 8192, 2048
+    lay = G.Layer(n, k, 4, 128, seed=0)
+    x = o.make_activations(m, k, seed=0)
+    y = lay.run(x)
+    rows = np.array([0, 1, 777, 2047])
+    G.assert_close_to_oracle(y[rows], x[rows], lay.w, "70B o-proj prefill")
+    # every row agrees with the decode kernel run on that row alone (different kernel, same answer)
+    y1 = lay.run(x[5:6])
+    assert np.max(np.abs(y1.astype(np.float64) - y[5:6])) <= 2e-3 * np.max(np.abs(y1.astype(np.float64)))
+
+
+def test_sync_flag_and_error_paths_on_device():
+    lay = G.Layer(32, 256, 4, 128, seed=1)
+    x = o.make_activations(2, 256, seed=1)
+    y_async = lay.run(x, flags=1)
+    y_sync = lay.run(x, flags=0)  # SYNC: the call itself waits for the kernel
+    assert np.array_equal(y_async, y_sync)
+    with pytest.raises(_lib.MatGPTQError, match="variant"):
+        lay.run(x, flags=1 | (200 << 8))
+    with pytest.raises(_lib.MatGPTQError, match="bfloat16"):
+        lay.run(x, flags=3)

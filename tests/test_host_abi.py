@@ -1,0 +1,133 @@
+"""C ABI on the host: every declared symbol is exported, the packers round-trip, the
+size contract of the reference's op holds, errors come back as codes.  No GPU work."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+from hypothesis import given, settings, strategies as st
+
+from matgptq_amd import _lib
+from oracle import matgptq_oracle as o
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BITS = (2, 3, 4, 6, 8)
+
+
+def L():
+    return _lib.load()
+
+
+def test_every_declared_symbol_is_exported():
+    header = open(os.path.join(ROOT, "include", "matgptq_abi.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    names = set(re.findall(r"\b(matgptq_[a-z_0-9]+)\s*\(", header))
+    assert names == set(_lib.EXPORTS)
+    lib = ctypes.CDLL(_lib.ABI_PATH)
+    for n in sorted(names):
+        assert hasattr(lib, n), n
+    assert L().matgptq_abi_version() == 1
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_packed_size_contract(b):
+    # bitwidth * N * K / 32 words (inference_lib/matgptq_cuda/csrc/bindings.cpp:68,160)
+    for n, k in ((16, 128), (4096, 4096), (28672, 4096)):
+        assert L().matgptq_packed_words(b, n, k) == b * n * k // 32
+    assert L().matgptq_packed_words(5, 16, 128) == 0
+
+
+def _pack(codes, b, slice_=0):
+    n, k = codes.shape
+    out = np.zeros(L().matgptq_packed_words(b, n, k), dtype=np.uint32)
+    _lib.check(L().matgptq_pack_host(codes.ctypes.data, n, k, b, slice_, out.ctypes.data))
+    return out
+
+
+def _unpack(packed, n, k, b):
+    out = np.zeros((n, k), dtype=np.uint8)
+    _lib.check(L().matgptq_unpack_host(packed.ctypes.data, n, k, b, out.ctypes.data))
+    return out
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_pack_unpack_identity(b):
+    rng = np.random.default_rng(b)
+    for n, k in ((16, 128), (48, 384), (64, 1024)):
+        c = rng.integers(0, 1 << b, (n, k), dtype=np.uint8)
+        assert np.array_equal(_unpack(_pack(c, b), n, k, b), c)
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_pack_every_position_is_independent(b):
+    # a single non-zero code anywhere in a tile comes back alone: catches overlapping fields
+    top = (1 << b) - 1
+    for pos in range(0, 16 * 128, 37):
+        c = np.zeros((16, 128), dtype=np.uint8)
+        c[pos // 128, pos % 128] = top
+        assert np.array_equal(_unpack(_pack(c, b), 16, 128, b), c)
+
+
+@settings(max_examples=30, deadline=None)
+@given(st.sampled_from(BITS), st.integers(1, 3), st.integers(1, 3), st.integers(0, 2 ** 31 - 1))
+def test_pack_unpack_identity_property(b, nb, kb, seed):
+    rng = np.random.default_rng(seed)
+    c = rng.integers(0, 1 << b, (16 * nb, 128 * kb), dtype=np.uint8)
+    assert np.array_equal(_unpack(_pack(c, b), 16 * nb, 128 * kb, b), c)
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_pack_from_master_slices_like_the_oracle(b):
+    rng = np.random.default_rng(100 + b)
+    q = rng.integers(0, 256, (32, 256), dtype=np.uint8)
+    assert np.array_equal(_unpack(_pack(q, b, 1), 32, 256, b), o.slice_codes(q, b))
+    # all 256 master codes in one tile
+    q = np.tile(np.arange(256, dtype=np.uint8), 8).reshape(16, 128)
+    assert np.array_equal(_unpack(_pack(q, b, 1), 16, 128, b), o.slice_codes(q, b))
+
+
+def test_pack_ignores_bits_above_the_bitwidth():
+    rng = np.random.default_rng(9)
+    c = rng.integers(0, 256, (16, 128), dtype=np.uint8)
+    for b in (2, 3, 4, 6):
+        assert np.array_equal(_unpack(_pack(c, b), 16, 128, b), c & ((1 << b) - 1))
+
+
+@pytest.mark.parametrize("g", (128, 32, -1))
+def test_reorder_scales_is_the_tile_transpose(g):
+    n, k = 48, 512
+    G = 1 if g == -1 else k // g
+    s = np.arange(n * G, dtype=np.uint16).reshape(n, G)
+    out = np.zeros_like(s)
+    _lib.check(L().matgptq_reorder_scales_host(s.ctypes.data, n, k, g, out.ctypes.data))
+    expect = s.reshape(n // 16, 16, G).transpose(0, 2, 1)
+    assert np.array_equal(out.reshape(n // 16, G, 16), expect)
+
+
+def test_error_codes():
+    buf = np.zeros(16 * 128, dtype=np.uint8)
+    out = np.zeros(8 * 16 * 128 // 32, dtype=np.uint32)
+    lib = L()
+    assert lib.matgptq_pack_host(buf.ctypes.data, 16, 128, 5, 0, out.ctypes.data) == -1
+    assert lib.matgptq_pack_host(buf.ctypes.data, 15, 128, 4, 0, out.ctypes.data) == -3
+    assert lib.matgptq_pack_host(buf.ctypes.data, 16, 64, 4, 0, out.ctypes.data) == -3
+    assert lib.matgptq_pack_host(None, 16, 128, 4, 0, out.ctypes.data) == -4
+    assert lib.matgptq_reorder_scales_host(buf.ctypes.data, 16, 128, 64, out.ctypes.data) == -2
+    # argument checks of the GEMM come before any device work
+    assert lib.matgptq_gemm(4, 128, 16, 128, 1, None, None, None, None, None, None, 1) == -4
+    assert lib.matgptq_gemm(7, 128, 16, 128, 1, 1, 1, None, 1, 1, None, 1) == -1
+    assert lib.matgptq_gemm(4, 48, 16, 128, 1, 1, 1, None, 1, 1, None, 1) == -2
+    assert lib.matgptq_gemm(4, 128, 16, 128, 0, 1, 1, None, 1, 1, None, 1) == -8
+    assert lib.matgptq_gemm(4, 128, 16, 128, 1, 1, 1, None, 1, 1, None, 3) == -5  # bf16
+    for code in range(-8, 1):
+        assert lib.matgptq_strerror(code)
+    with pytest.raises(_lib.MatGPTQError, match="bitwidth must be one of"):
+        _lib.check(-1)
+
+
+def test_describe_plan_regimes():
+    assert _lib.describe_plan(4, 128, 4096, 4096, 1).startswith("decode")
+    assert _lib.describe_plan(4, 128, 4096, 4096, 16, True).startswith("decode")
+    assert _lib.describe_plan(4, 128, 8192, 8192, 2048).startswith("prefill")
+    assert _lib.describe_plan(3, 32, 16, 1024, 17).startswith("prefill")
