@@ -52,13 +52,14 @@ unpack_kernel(const uint32_t* __restrict__ packed, uint8_t* __restrict__ codes, 
   const int64_t tile = slot >> 6;
   const int64_t rb = tile / k_tiles, kb = tile - rb * k_tiles;
   const int r = lane & 15, q = lane >> 4;
+  const UnpackConsts<BITS> kc_unpack;
   uint32_t w[BITS];
   load_tile_words<BITS>(packed + tile * tile_words(BITS), lane, w);
   uint8_t* row = codes + (rb * 16 + r) * K + kb * 128 + q * 8;
   auto emit = [&](auto jtag) {
     constexpr int J = decltype(jtag)::value;
     uint32_t raw[4];
-    raw_octet<BITS, J>(w, raw);
+    raw_octet<BITS, J>(w, kc_unpack, raw);
     uint32_t lo = 0, hi = 0;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
@@ -111,13 +112,14 @@ dequant_kernel(const uint32_t* __restrict__ packed, const uint16_t* __restrict__
   const int64_t tile = slot >> 6;
   const int64_t rb = tile / k_tiles, kb = tile - rb * k_tiles;
   const int r = lane & 15, q = lane >> 4;
+  const UnpackConsts<BITS> kc_unpack;
   uint32_t w[BITS];
   load_tile_words<BITS>(packed + tile * tile_words(BITS), lane, w);
   _Float16* row = reinterpret_cast<_Float16*>(w_out) + (rb * 16 + r) * K + kb * 128 + q * 8;
   auto emit = [&](auto jtag) {
     constexpr int J = decltype(jtag)::value;
     uint32_t raw[4];
-    raw_octet<BITS, J>(w, raw);
+    raw_octet<BITS, J>(w, kc_unpack, raw);
     const int64_t k0 = kb * 128 + J * 32 + q * 8;
     const int64_t g = group_size == -1 ? 0 : k0 / group_size;
     const size_t so = ((size_t)rb * G + g) * 16 + r;

@@ -104,6 +104,7 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
 
   using StageT = Stage<BITS, R, U, GPT, ZP>;
   StageT cur, nxt;
+  const UnpackConsts<BITS> kc_unpack;
 
   // loads stage `stage` of chunk [c0, c1) of the row blocks starting at rb0
   auto load_stage = [&](StageT& st, int rb0, int c0, int c1, int stage) {
@@ -190,7 +191,7 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
       Frag aw;
-      raw_octet<BITS, J>(st.w[u][rr], aw.u);
+      raw_octet<BITS, J>(st.w[u][rr], kc_unpack, aw.u);
       // a group's first product starts from a zero accumulator operand
       constexpr bool kFresh = GROUP == 32 || (GROUP == 128 && J == 0);
       const float4v zero4 = {0.f, 0.f, 0.f, 0.f};

@@ -55,19 +55,47 @@ __device__ __forceinline__ half2v centre_raw(uint32_t raw, int centre) {
   }
 }
 
-// (x & mask) | orv in one VALU instruction.  `mask` travels in an SGPR and `orv`
-// in a VGPR: a VOP3 encoding of this target takes no literal and one scalar operand.
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t orv) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(orv));
-  return r;
+// (x & mask) | orv.  The compiler folds this into one v_and_or_b32 when neither constant
+// is a literal: a VOP3 encoding of this target takes no literal and one scalar operand.
+// `opaque_*` hide a constant's value from the optimiser (no instruction is emitted), so the
+// mask stays in an SGPR and the OR-ed word in a VGPR.  The instruction itself is chosen by
+// the compiler, which keeps its hazard bookkeeping (VALU result -> MFMA operand) intact.
+__device__ __forceinline__ uint32_t opaque_sgpr(uint32_t v) {
+  asm("" : "+s"(v));
+  return v;
 }
+__device__ __forceinline__ uint32_t opaque_vgpr(uint32_t v) {
+  asm("" : "+v"(v));
+  return v;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t orv) {
+  return (x & mask) | orv;
+}
+
+// The constants of the unpack sequence, made opaque once per kernel.
+template <int BITS>
+struct UnpackConsts {
+  uint32_t magic;  // VGPR: two fp16 1024.0
+  uint32_t m[3];   // SGPRs: field masks
+  __device__ __forceinline__ UnpackConsts() {
+    magic = opaque_vgpr(kMagic);
+    if constexpr (BITS == 2) {
+      m[0] = opaque_sgpr(0x00030003u); m[1] = opaque_sgpr(0x000C000Cu); m[2] = opaque_sgpr(0x00300030u);
+    } else if constexpr (BITS == 6) {
+      m[0] = opaque_sgpr(0x00030003u); m[1] = opaque_sgpr(0x00300030u); m[2] = 0;
+    } else if constexpr (BITS == 3) {
+      m[0] = opaque_sgpr(0x000F000Fu); m[1] = opaque_sgpr(0x00F000F0u); m[2] = opaque_sgpr(0x44444444u);
+    } else {
+      m[0] = opaque_sgpr(0x000F000Fu); m[1] = opaque_sgpr(0x00F000F0u); m[2] = 0;
+    }
+  }
+};
 
 // Device form of Codec<BITS>::decode_octet (same results, fewer instructions):
 // the four raw pairs 1024 + c * 2^p of octet J.
 template <int BITS, int J>
-__device__ __forceinline__ void raw_octet(const uint32_t (&w)[BITS], uint32_t (&r)[4]) {
-  const uint32_t magic = kMagic;
+__device__ __forceinline__ void raw_octet(const uint32_t (&w)[BITS], const UnpackConsts<BITS>& k,
+                                          uint32_t (&r)[4]) {
   if constexpr (BITS == 4 || BITS == 3) {
     uint32_t x;
     if constexpr (BITS == 4) {
@@ -76,36 +104,36 @@ __device__ __forceinline__ void raw_octet(const uint32_t (&w)[BITS], uint32_t (&
       const uint32_t lo = (w[J >> 1] >> (2 * (J & 1))) & 0x33333333u;
       const uint32_t c = w[2];
       const uint32_t cs = J == 0 ? (c << 2) : J == 1 ? (c << 1) : J == 2 ? c : (c >> 1);
-      x = and_or(cs, 0x44444444u, lo);
+      x = and_or(cs, k.m[2], lo);
     }
     const uint32_t x8 = x >> 8;
-    r[0] = and_or(x, 0x000F000Fu, magic);
-    r[1] = and_or(x, 0x00F000F0u, magic);
-    r[2] = and_or(x8, 0x000F000Fu, magic);
-    r[3] = and_or(x8, 0x00F000F0u, magic);
+    r[0] = and_or(x, k.m[0], k.magic);
+    r[1] = and_or(x, k.m[1], k.magic);
+    r[2] = and_or(x8, k.m[0], k.magic);
+    r[3] = and_or(x8, k.m[1], k.magic);
   } else if constexpr (BITS == 2) {
     const uint32_t x = w[J >> 1];
     const uint32_t x6 = x >> 6;
     if constexpr ((J & 1) == 0) {
-      r[0] = and_or(x, 0x00030003u, magic);
-      r[1] = and_or(x, 0x000C000Cu, magic);
-      r[2] = and_or(x, 0x00300030u, magic);
-      r[3] = and_or(x6, 0x00030003u, magic);
+      r[0] = and_or(x, k.m[0], k.magic);
+      r[1] = and_or(x, k.m[1], k.magic);
+      r[2] = and_or(x, k.m[2], k.magic);
+      r[3] = and_or(x6, k.m[0], k.magic);
     } else {
       const uint32_t x12 = x >> 12;
-      r[0] = and_or(x6, 0x000C000Cu, magic);
-      r[1] = and_or(x6, 0x00300030u, magic);
-      r[2] = and_or(x12, 0x00030003u, magic);
-      r[3] = and_or(x12, 0x000C000Cu, magic);
+      r[0] = and_or(x6, k.m[1], k.magic);
+      r[1] = and_or(x6, k.m[2], k.magic);
+      r[2] = and_or(x12, k.m[0], k.magic);
+      r[3] = and_or(x12, k.m[1], k.magic);
     }
   } else if constexpr (BITS == 6) {
     const uint32_t h = w[J], h8 = h >> 8;
     const uint32_t l = (J & 1) ? (w[4 + (J >> 1)] >> 8) : w[4 + (J >> 1)];
     const uint32_t l2 = l >> 2;
-    r[0] = ((h & 0x000F000Fu) << 2) | and_or(l, 0x00030003u, magic);
-    r[1] = ((h & 0x00F000F0u) << 2) | and_or(l, 0x00300030u, magic);
-    r[2] = ((h8 & 0x000F000Fu) << 2) | and_or(l2, 0x00030003u, magic);
-    r[3] = ((h8 & 0x00F000F0u) << 2) | and_or(l2, 0x00300030u, magic);
+    r[0] = ((h & 0x000F000Fu) << 2) | and_or(l, k.m[0], k.magic);
+    r[1] = ((h & 0x00F000F0u) << 2) | and_or(l, k.m[1], k.magic);
+    r[2] = ((h8 & 0x000F000Fu) << 2) | and_or(l2, k.m[0], k.magic);
+    r[3] = ((h8 & 0x00F000F0u) << 2) | and_or(l2, k.m[1], k.magic);
   } else {
     // bytes: pair 2d = (byte0, byte2) of word 2J+d, pair 2d+1 = (byte1, byte3)
     const uint32_t fill = 0x64646464u;
@@ -118,9 +146,10 @@ __device__ __forceinline__ void raw_octet(const uint32_t (&w)[BITS], uint32_t (&
 
 // Octet j of a lane -> MFMA operand holding (c - 2^(b-1)) for its eight codes.
 template <int BITS, int J>
-__device__ __forceinline__ void centred_octet(const uint32_t (&w)[BITS], Frag& a) {
+__device__ __forceinline__ void centred_octet(const uint32_t (&w)[BITS], const UnpackConsts<BITS>& k,
+                                              Frag& a) {
   uint32_t raw[4];
-  raw_octet<BITS, J>(w, raw);
+  raw_octet<BITS, J>(w, k, raw);
   constexpr int c = Codec<BITS>::kCentre;
   a.p[0] = centre_raw<Codec<BITS>::raw_shift(J, 0)>(raw[0], c);
   a.p[1] = centre_raw<Codec<BITS>::raw_shift(J, 1)>(raw[1], c);

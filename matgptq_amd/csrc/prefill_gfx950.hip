@@ -48,10 +48,10 @@ __device__ __forceinline__ half2v dequant_pair(uint32_t raw, half2v zrel, half2v
 }
 
 template <int BITS, int J, bool ZP>
-__device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], half2v zrel, half2v scale,
-                                              Frag& a) {
+__device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const UnpackConsts<BITS>& k,
+                                              half2v zrel, half2v scale, Frag& a) {
   uint32_t raw[4];
-  raw_octet<BITS, J>(w, raw);
+  raw_octet<BITS, J>(w, k, raw);
   a.p[0] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 0), ZP>(raw[0], zrel, scale);
   a.p[1] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 1), ZP>(raw[1], zrel, scale);
   a.p[2] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 2), ZP>(raw[2], zrel, scale);
@@ -92,6 +92,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[rr][mt] = float4v{0.f, 0.f, 0.f, 0.f};
 
+  const UnpackConsts<BITS> kc_unpack;
   uint32_t wcur[RBW][BITS], wnxt[RBW][BITS];
   _Float16 scur[RBW][GPT], snxt[RBW][GPT];
   _Float16 zcur[RBW][GPT], znxt[RBW][GPT];
@@ -155,9 +156,9 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
         half2v zr = {(_Float16)0.f, (_Float16)0.f};
         if constexpr (ZP) zr = half2v{zcur[rr][gg], zcur[rr][gg]};
         if (jj == 0)
-          dequant_octet<BITS, J0, ZP>(wcur[rr], zr, sc, aw[rr]);
+          dequant_octet<BITS, J0, ZP>(wcur[rr], kc_unpack, zr, sc, aw[rr]);
         else
-          dequant_octet<BITS, J0 + 1, ZP>(wcur[rr], zr, sc, aw[rr]);
+          dequant_octet<BITS, J0 + 1, ZP>(wcur[rr], kc_unpack, zr, sc, aw[rr]);
       }
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
