@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the bit-sliced GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+One STEP is one pass of the decode hot path over the four Llama-3-8B-shaped linears
+(qkv 4096->6144, o 4096->4096, gate_up 4096->28672, down 14336->4096) at batch 1,
+weights sliced to 4 bits, group 128, fp16 scale and zero per group (the zero-point form).
+`value` is the sliced weight bytes of a step divided by its time (GB/s): the figure the
+HBM roofline is quoted on.  Inputs are resident in HBM before the timed region; every
+step reads a different copy of the weights, cycling through a ring of copies larger
+than 2 GiB so that the 256 MB Infinity Cache cannot serve them.
+
+The JSON line also carries
+  roofline     the dominant kernel (gate_up decode) alone: algorithmic bytes per launch /
+               average launch duration measured with HIP events on the launch stream
+  cpu_baseline the reference's PyTorch CPU path (slice -> dequantize -> F.linear,
+               restated in oracle/torch_path.py) on the host cores, same layers, one pass
+  extra        per-bitwidth / per-layer times, small-batch and M=2048 prefill figures
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix rate
+LLAMA3_8B = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "down": (4096, 14336)}
+LLAMA3_70B = {"qkv": (10240, 8192), "o": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
+GROUP = 128
+RING_BYTES = 2.5e9
+
+
+def algorithmic_bytes(n, k, m, bits, zero_points=True):
+    """Bytes a GEMV call must move: sliced codes + scales (+ zeros) + x + y."""
+    aux = 2 if zero_points else 1
+    return n * k * bits // 8 + 2 * n * (k // GROUP) * aux + 2 * m * k + 2 * m * n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from matgptq_amd import _lib
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X", file=sys.stderr)
+        return 2
+    L = _lib.load()  # raises if the HIP library is missing: there is no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.Stream(device=dev)  # default priority
+
+    def launch(bits, n, k, x, packed, scales, zeros, y, flags=1):
+        _lib.check(L.matgptq_gemm(bits, GROUP, n, k, x.shape[0], packed.data_ptr(), scales.data_ptr(),
+                                  zeros.data_ptr() if zeros is not None else None, x.data_ptr(),
+                                  y.data_ptr(), stream.cuda_stream, flags))
+
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def make_ring(n, k, bits, copies):
+        words = L.matgptq_packed_words(bits, n, k)
+        # random words are valid packed codes: every bit pattern decodes to some code
+        return [torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), dtype=torch.int32, device=dev, generator=g)
+                for _ in range(copies)]
+
+    def make_aux(n, k):
+        groups = n * (k // GROUP)
+        scales = (torch.randn(groups, device=dev, generator=g).abs() * 0.01 + 1e-3).to(torch.float16)
+        zeros = torch.randint(0, 256, (groups,), device=dev, generator=g).to(torch.float16)
+        return scales, zeros
+
+    def timed_graph(build, reps=3):
+        """Captures `build()` (launches on `stream`) into a HIP graph; returns the best
+        replay time in seconds, measured with events on `stream`."""
+        with torch.cuda.stream(stream):
+            build()  # eager warm-up of every kernel in the graph
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                build()
+            graph.replay()
+            stream.synchronize()
+            best = float("inf")
+            for _ in range(reps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                graph.replay()
+                e1.record(stream)
+                stream.synchronize()
+                best = min(best, e0.elapsed_time(e1) * 1e-3)
+        return best
+
+    # ------------------------------------------------------------------ headline
+    bits = 4
+    step_bytes = sum(n * k * bits // 8 for n, k in LLAMA3_8B.values())
+    copies = max(2, int(RING_BYTES // step_bytes) + 1)
+    rings = {name: make_ring(n, k, bits, copies) for name, (n, k) in LLAMA3_8B.items()}
+    aux = {name: make_aux(n, k) for name, (n, k) in LLAMA3_8B.items()}
+    xs = {name: torch.randn(1, k, device=dev, generator=g).to(torch.float16) for name, (n, k) in LLAMA3_8B.items()}
+    ys = {name: torch.empty(1, n, dtype=torch.float16, device=dev) for name, (n, k) in LLAMA3_8B.items()}
+
+    def step(i):
+        for name, (n, k) in LLAMA3_8B.items():
+            launch(bits, n, k, xs[name], rings[name][i % copies], aux[name][0], aux[name][1], ys[name])
+
+    with torch.cuda.stream(stream):
+        for i in range(args.warmup):
+            step(i)
+        stream.synchronize()
+    torch.cuda.synchronize()
+    t_wall0 = time.perf_counter()
+    elapsed = timed_graph(lambda: [step(i) for i in range(args.steps)], reps=1)
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter() - t_wall0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = step_bytes / (elapsed / args.steps) / 1e9
+
+    # --------------------------------------------------------- dominant kernel
+    n, k = LLAMA3_8B["gate_up"]
+    launches = max(copies, 64)
+    t_dom = timed_graph(lambda: [launch(bits, n, k, xs["gate_up"], rings["gate_up"][i % copies],
+                                        aux["gate_up"][0], aux["gate_up"][1], ys["gate_up"])
+                                 for i in range(launches)]) / launches
+    dom_bytes = algorithmic_bytes(n, k, 1, bits)
+    roofline = {
+        "kernel": _lib.describe_plan(bits, GROUP, n, k, 1, True),
+        "bound": "hbm",
+        "achieved": round(dom_bytes / t_dom / 1e9, 1),
+        "peak": HBM_PEAK_GBPS,
+        "unit": "GB/s",
+        "frac": round(dom_bytes / t_dom / 1e9 / HBM_PEAK_GBPS, 4),
+        "traffic": None,
+        "us_per_launch": round(t_dom * 1e6, 2),
+        "algorithmic_bytes": dom_bytes,
+    }
+
+    extra = {}
+    cpu_baseline = None
+    if not args.quick:
+        # ------------------------------------------------- per layer, per bitwidth
+        table = {}
+        for b in (8, 6, 4, 3, 2):
+            for name, (n, k) in LLAMA3_8B.items():
+                wbytes = n * k * b // 8
+                cp = max(2, int(RING_BYTES // wbytes) + 1)
+                ring = rings[name] if b == bits else make_ring(n, k, b, cp)
+                cp = len(ring)
+                reps = max(cp, 32)
+                for zp in (True, False):
+                    t = timed_graph(lambda: [launch(b, n, k, xs[name], ring[i % cp], aux[name][0],
+                                                    aux[name][1] if zp else None, ys[name])
+                                             for i in range(reps)]) / reps
+                    table[f"{name}_b{b}_{'zp' if zp else 'sym'}"] = {
+                        "us": round(t * 1e6, 2),
+                        "weight_GBps": round(wbytes / t / 1e9, 1),
+                        "pct_hbm_peak": round(wbytes / t / 1e9 / HBM_PEAK_GBPS * 100, 1),
+                    }
+                del ring
+        extra["gemv_M1"] = table
+        # ----------------------------------------------------------- small batch
+        small = {}
+        for m in (2, 4, 8, 16):
+            for b in (4, 3):
+                name = "gate_up"
+                n, k = LLAMA3_8B[name]
+                ring = rings[name] if b == bits else make_ring(n, k, b, max(2, int(RING_BYTES // (n * k * b // 8)) + 1))
+                cp = len(ring)
+                xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+                ym = torch.empty(m, n, dtype=torch.float16, device=dev)
+                t = timed_graph(lambda: [launch(b, n, k, xm, ring[i % cp], aux[name][0], aux[name][1], ym)
+                                         for i in range(cp)]) / cp
+                small[f"gate_up_b{b}_M{m}"] = {"us": round(t * 1e6, 2),
+                                               "weight_GBps": round(n * k * b / 8 / t / 1e9, 1)}
+        extra["small_batch"] = small
+        del rings
+        torch.cuda.empty_cache()
+        # --------------------------------------------------------------- prefill
+        pre = {}
+        m = 2048
+        for name, (n, k) in LLAMA3_70B.items():
+            packed = make_ring(n, k, 4, 1)[0]
+            sc, zr = make_aux(n, k)
+            xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+            ym = torch.empty(m, n, dtype=torch.float16, device=dev)
+            for zp in (True, False):
+                t = timed_graph(lambda: [launch(4, n, k, xm, packed, sc, zr if zp else None, ym) for _ in range(5)]) / 5
+                tf = 2.0 * m * n * k / t / 1e12
+                pre[f"{name}_b4_M2048_{'zp' if zp else 'sym'}"] = {
+                    "ms": round(t * 1e3, 3), "TFLOPs": round(tf, 1),
+                    "pct_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS * 100, 1)}
+            del packed, xm, ym
+        extra["prefill_llama3_70b"] = pre
+        # ---------------------------------------------------------- CPU baseline
+        cpu_baseline = cpu_path_baseline(step_bytes)
+
+    out = {
+        "metric": "batch1_gemv_sliced_weight_GBps_4bit_llama3_8b_layers",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: Llama-3-8B linears qkv/o/gate_up/down, M=1 decode, 4-bit slice, "
+                               "group 128, fp16 scale+zero; ring of weight copies > 2 GiB",
+                   "pct_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 1),
+                   "wall_s_timed_region": round(t_wall, 4)},
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+def cpu_path_baseline(step_bytes: int):
+    """One pass of the same four layers through the reference's CPU PyTorch path."""
+    import torch
+
+    from oracle import torch_path
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    gen = torch.Generator().manual_seed(0)
+    layers = []
+    for name, (n, k) in LLAMA3_8B.items():
+        q = torch.randint(0, 256, (n, k), dtype=torch.uint8, generator=gen)
+        s = (torch.randn(n, k // GROUP, generator=gen).abs() * 0.01 + 1e-3).to(torch.float16)
+        z = torch.randint(0, 256, (n, k // GROUP), generator=gen).to(torch.float16)
+        x = torch.randn(1, k, generator=gen).to(torch.float16)
+        layers.append((q, s, z, x))
+    with torch.no_grad():
+        q, s, z, x = layers[1]
+        torch_path.forward(x, q, s, z, 8, 4)  # warm-up on the smallest layer
+        best = float("inf")
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for q, s, z, x in layers:
+                torch_path.forward(x, q, s, z, 8, 4)
+            best = min(best, time.perf_counter() - t0)
+    return {
+        "value": round(step_bytes / best / 1e9, 3),
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"one full step (4 layers, M=1, 4-bit), best of 5, {best:.3f} s per step: "
+                  "slice + dequantize + F.linear in torch on the host, fp16",
+    }
+
+
+if __name__ == "__main__":
+    sys.exit(main())
