@@ -16,7 +16,7 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
 
 #define MATGPTQ_DECL(B)                                                                        \
   hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int S, int W, int kc,  \
-                                int max_wgs, bool stream_flavour, size_t smem, hipStream_t);   \
+                                bool stream_flavour, size_t smem, hipStream_t);                \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);
 MATGPTQ_DECL(2)
 MATGPTQ_DECL(3)
@@ -41,7 +41,6 @@ struct Plan {
   bool decode;
   int R, S, W;   // decode: row blocks per wave, slots and k-slices per workgroup
   int kc;        // decode: tiles of K staged in LDS at a time
-  int max_wgs;   // decode: grid cap (0 = none)
   bool stream;   // decode: double-buffered flavour
   size_t smem;   // decode: dynamic LDS bytes
   int cfg;       // prefill: tile configuration
@@ -58,39 +57,23 @@ size_t decode_lds_bytes(int R, int S, int W, int kc, int64_t M) {
   return (size_t)S * W * R * 1024 + (size_t)M * ((size_t)kc * 128 + 8) * 2;
 }
 
-int device_cu_count() {
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      cus = n;
-    else
-      cus = 256;
-  }
-  return cus;
-}
-
 // Automatic choice; the flags word can override it for benchmarks:
 //   bits 8..15 : 0 = automatic, 1 + rsel + 3*shape = decode (rsel: R = 1,2,4; shape: kShapes),
 //                64 + cfg = prefill tile configuration
 //   bits 16..17: decode flavour, 0 = automatic, 1 = burst, 2 = stream
-//   bits 18..20: decode grid cap, 0 = automatic, 1 = none, n >= 2: (n-1) workgroups per CU
 int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp, uint32_t flags,
               Plan* p) {
   const int row_blocks = (int)(N / 16), k_tiles = (int)(K / 128);
   const int variant = (int)((flags & MATGPTQ_FLAG_VARIANT_MASK) >> MATGPTQ_FLAG_VARIANT_SHIFT);
   const int flavour = (int)((flags >> 16) & 3u);
-  const int cap_sel = (int)((flags >> 18) & 7u);
   p->decode = M <= kDecodeMaxM;
   p->cfg = 0;
   // default decode shape (measured on MI355X, M = 1, Llama-3-8B layers): eight waves per
-  // workgroup; few row blocks -> all eight split K, many -> two slots of four k-slices;
-  // two row blocks per wave once there are enough of them to keep the grid wide
+  // workgroup, all of them splitting K; four row blocks per wave once there are enough
+  // row blocks to keep every CU busy that way
   int W = 8, S = 1;
-  if (row_blocks >= 1024) { W = 4; S = 2; }
   while (W > 1 && W > k_tiles) { W >>= 1; S <<= 1; }
-  int R = (row_blocks >= 320 && row_blocks % 2 == 0) ? 2 : 1;
+  int R = row_blocks >= 1024 ? 4 : 1;
   // default prefill tile
   if (!p->decode) {
     if (M <= 32) p->cfg = 4;
@@ -117,7 +100,6 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     p->R = p->S = p->W = p->kc = 0;
     p->stream = false;
     p->smem = 0;
-    p->max_wgs = 0;
     return MATGPTQ_OK;
   }
   // burst keeps at most eight waves per workgroup; long tile runs prefer stream
@@ -138,9 +120,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   p->kc = (int)kc;
   p->stream = stream;
   p->smem = decode_lds_bytes(R, S, W, (int)kc, M);
-  // a capped grid only pays when X' is staged once (kc covers K)
-  p->max_wgs = 0;
-  if (kc >= k_tiles && cap_sel >= 2) p->max_wgs = (cap_sel - 1) * device_cu_count();
+  if (kc < k_tiles && S * W > 8) return variant != 0 ? MATGPTQ_EVARIANT : MATGPTQ_ESIZE;
   (void)zp;
   (void)group_size;
   (void)bits;
@@ -149,11 +129,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
 
 hipError_t launch_decode(int bits, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
   switch (bits) {
-    case 2: return launch_decode_b2(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
-    case 3: return launch_decode_b3(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
-    case 4: return launch_decode_b4(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
-    case 6: return launch_decode_b6(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
-    default: return launch_decode_b8(a, g, p.R, p.S, p.W, p.kc, p.max_wgs, p.stream, p.smem, s);
+    case 2: return launch_decode_b2(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
+    case 3: return launch_decode_b3(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
+    case 4: return launch_decode_b4(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
+    case 6: return launch_decode_b6(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
+    default: return launch_decode_b8(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
   }
 }
 
@@ -232,9 +212,9 @@ int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, in
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, has_zeros != 0, flags, &p)) return e;
   if (p.decode)
-    snprintf(buf, buf_len, "decode-%s b%d g%d zp%d R%d S%d W%d kc%d cap%d lds%zu",
-             p.stream ? "stream" : "burst", bitwidth, group_size, has_zeros ? 1 : 0, p.R, p.S, p.W,
-             p.kc, p.max_wgs, p.smem);
+    snprintf(buf, buf_len, "decode-%s b%d g%d zp%d R%d S%d W%d kc%d lds%zu",
+             p.kc < (int)(K / 128) ? "chunked" : (p.stream ? "stream" : "burst"), bitwidth, group_size,
+             has_zeros ? 1 : 0, p.R, p.S, p.W, p.kc, p.smem);
   else
     snprintf(buf, buf_len, "prefill b%d g%d zp%d cfg%d", bitwidth, group_size, has_zeros ? 1 : 0,
              p.cfg);

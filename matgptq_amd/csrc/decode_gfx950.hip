@@ -21,11 +21,9 @@
 //     D -= (zero-128)/2^(8-b) 2^p * X' (one value per row and group, zero-point form only)
 // so D = sum_k ((c << (8-b)) - zero) x / 2^(8-b) over the group, exact products.
 // Per group the fp32 D is multiplied by the group scale in fp32 and added to
-// the running sum; 2^(8-b) is applied to the final value.
-//
-// Persistence.  When all of X' fits in LDS the grid may be capped: a workgroup then
-// stages X' once and walks several groups of row blocks, with the first loads of the
-// next group in flight while the sums of the current one are combined and stored.
+// the running sum; 2^(8-b) is applied to the final value.  The constant-operand chain
+// does not depend on the row, so it is computed once per tile and the chains of the R
+// row blocks of a wave start from it.
 #include "device_common.h"
 
 #ifndef MATGPTQ_BITS
@@ -56,10 +54,9 @@ __device__ __forceinline__ half2v inv_pow_pair() {
 }
 
 struct DecodeShape {
-  int S, W;       // slots and k-slices per workgroup
-  int kc;         // tiles of K whose activations are staged in LDS at a time
-  int n_groups;   // groups of S*R row blocks; workgroups walk them with stride gridDim.x
-  int lg_rows;    // log2(S * R * 16)
+  int S, W;     // slots and k-slices per workgroup
+  int kc;       // tiles of K whose activations are staged in LDS at a time
+  int lg_rows;  // log2(S * R * 16)
 };
 
 template <int BITS, int R, int U, int GPT, bool ZP>
@@ -69,7 +66,8 @@ struct Stage {
   _Float16 z[ZP ? U : 1][R][GPT];  // zero of row lane%16 (operand layout)
 };
 
-template <int BITS, int GROUP, bool ZP, int R, bool STREAM>
+// STREAM: double-buffered stages.  CHUNKED: X' is staged kc tiles at a time.
+template <int BITS, int GROUP, bool ZP, int R, bool STREAM, bool CHUNKED>
 __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape sh) {
   constexpr int U = tiles_in_flight(BITS, R);
   constexpr bool GROUPED = GROUP != -1;
@@ -85,6 +83,9 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
   const int ws = wave - slot * W;
   const int r16 = lane & 15;  // row of the weight operand / batch column of the x operand
   const int q = lane >> 4;
+  const int rb_wg = blockIdx.x * S * R;  // first row block of the workgroup
+  const int rb0 = rb_wg + slot * R;      // first row block of this wave
+  const bool live = rb0 < a.row_blocks;  // the last workgroup may have idle slots
 
   // LDS: [ partial sums | X' ]
   float* red = reinterpret_cast<float*>(smem);                                  // [S*W][R][256]
@@ -100,14 +101,13 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
   const BufRsrc wres = make_rsrc(a.packed, (uint32_t)a.row_blocks * rb_bytes);
   const BufRsrc sres = make_rsrc(a.scales, aux_bytes);
   const BufRsrc zres = make_rsrc(ZP ? a.zeros : a.scales, aux_bytes);
-  const bool single = kc >= a.k_tiles;  // all of X' fits: staged once per workgroup
 
   using StageT = Stage<BITS, R, U, GPT, ZP>;
   StageT cur, nxt;
   const UnpackConsts<BITS> kc_unpack;
 
-  // loads stage `stage` of chunk [c0, c1) of the row blocks starting at rb0
-  auto load_stage = [&](StageT& st, int rb0, int c0, int c1, int stage) {
+  // loads stage `stage` of chunk [c0, c1): tiles c0 + ws + W * (stage * U + u)
+  auto load_stage = [&](StageT& st, int c0, int c1, int stage) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int t = c0 + ws + W * (stage * U + u);
@@ -163,196 +163,220 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
   };
 
   float4v acc[R];  // sum over groups of scale * D
-  float4v d[R];    // running group sum
+  float4v d[R];    // running group sum (g = -1: running sum without the offset term)
+  float4v db;      // offset term of the running sum, g = -1 only
+#pragma unroll
+  for (int rr = 0; rr < R; rr++) {
+    acc[rr] = float4v{0.f, 0.f, 0.f, 0.f};
+    d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
+  }
+  db = float4v{0.f, 0.f, 0.f, 0.f};
+  _Float16 zrow[R];  // g = -1: zero of this lane's row
+  if constexpr (!GROUPED && ZP) {
+#pragma unroll
+    for (int rr = 0; rr < R; rr++)
+      zrow[rr] = live ? reinterpret_cast<const _Float16*>(a.zeros)[(size_t)(rb0 + rr) * 16 + r16]
+                      : (_Float16)128.0f;
+  }
 
-  auto fold_group = [&](const uint2 s4, int rr) {
+  auto fold = [&](const uint2 s4, int rr, const float4v v) {
     H4 s;
     s.v = s4;
 #pragma unroll
-    for (int i = 0; i < 4; i++) acc[rr][i] += (float)s.h[i] * d[rr][i];
+    for (int i = 0; i < 4; i++) acc[rr][i] += (float)s.h[i] * v[i];
   };
 
-  auto octet_step = [&](const StageT& st, int u, int tl, auto jtag) {  // tl: tile index inside the LDS copy
+  const float4v zero4 = {0.f, 0.f, 0.f, 0.f};
+
+  // constant operand -(1024 + centre * 2^p): removes the magic offset and centres the codes
+  auto bias_operand = [&](auto jtag) {
     constexpr int J = decltype(jtag)::value;
-#ifdef MATGPTQ_DEBUG_NOCOMPUTE
-    for (int rr = 0; rr < R; rr++) acc[rr][0] += __uint_as_float(st.w[u][rr][J % BITS] & 0x3f000000u);
-    if (tl < 0) acc[0][1] += (float)xb[tl];
-    return;
-#endif
-    Frag b;
-    b.v = *reinterpret_cast<const uint4*>(xb + tl * 128 + J * 32);
-    // constant operand  -(1024 + centre * 2^p)
-    Frag bias;
     constexpr float cc = (float)Codec<BITS>::kCentre;
+    Frag bias;
     bias.p[0] = h2_splat(-1024.0f) - pow_pair<BITS, J, 0>(cc);
     bias.p[1] = h2_splat(-1024.0f) - pow_pair<BITS, J, 1>(cc);
     bias.p[2] = h2_splat(-1024.0f) - pow_pair<BITS, J, 2>(cc);
     bias.p[3] = h2_splat(-1024.0f) - pow_pair<BITS, J, 3>(cc);
+    return bias;
+  };
+  // operand -(zero - 128) / 2^(8-b) * 2^p for this lane's row: exact in fp16
+  auto zero_operand = [&](_Float16 zv, auto jtag) {
+    constexpr int J = decltype(jtag)::value;
+    const _Float16 zrel = (_Float16)128.0f - zv;
+    const half2v z2 = {zrel, zrel};
+    Frag az;
+    az.p[0] = z2 * pow_pair<BITS, J, 0>(1.0f / kMul);
+    az.p[1] = z2 * pow_pair<BITS, J, 1>(1.0f / kMul);
+    az.p[2] = z2 * pow_pair<BITS, J, 2>(1.0f / kMul);
+    az.p[3] = z2 * pow_pair<BITS, J, 3>(1.0f / kMul);
+    return az;
+  };
+  auto raw_operand = [&](const StageT& st, int u, int rr, auto jtag) {
+    constexpr int J = decltype(jtag)::value;
+    Frag aw;
+    raw_octet<BITS, J>(st.w[u][rr], kc_unpack, aw.u);
+    return aw;
+  };
+#define MATGPTQ_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16((A).h, (B).h, (C), 0, 0, 0)
+
+  // One tile (tl = its index inside the LDS copy of X').  The offset chain does not depend
+  // on the row, so it is computed once and every row block's chain starts from it.
+  auto tile_step = [&](const StageT& st, int u, int tl) {
+    using J0 = std::integral_constant<int, 0>;
+    using J1 = std::integral_constant<int, 1>;
+    using J2 = std::integral_constant<int, 2>;
+    using J3 = std::integral_constant<int, 3>;
+#ifdef MATGPTQ_DEBUG_NOCOMPUTE
+    for (int rr = 0; rr < R; rr++)
+      for (int j = 0; j < BITS; j++) acc[rr][0] += __uint_as_float(st.w[u][rr][j] & 0x3f000000u);
+    if (tl < 0) acc[0][1] += (float)xb[tl];
+    return;
+#endif
+    Frag b[4];
 #pragma unroll
-    for (int rr = 0; rr < R; rr++) {
-      Frag aw;
-      raw_octet<BITS, J>(st.w[u][rr], kc_unpack, aw.u);
-      // a group's first product starts from a zero accumulator operand
-      constexpr bool kFresh = GROUP == 32 || (GROUP == 128 && J == 0);
-      const float4v zero4 = {0.f, 0.f, 0.f, 0.f};
-      d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw.h, b.h, kFresh ? zero4 : d[rr], 0, 0, 0);
-      d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bias.h, b.h, d[rr], 0, 0, 0);
-      if constexpr (ZP) {
-        // -(zero - 128) / 2^(8-b) * 2^p for this lane's row: exact in fp16
-        _Float16 zv;
-        if constexpr (GROUPED) zv = st.z[u][rr][GROUP == 32 ? J : 0];
-        else zv = st.z[0][rr][0];
-        const _Float16 zrel = (_Float16)128.0f - zv;
-        const half2v z2 = {zrel, zrel};
-        Frag az;
-        az.p[0] = z2 * pow_pair<BITS, J, 0>(1.0f / kMul);
-        az.p[1] = z2 * pow_pair<BITS, J, 1>(1.0f / kMul);
-        az.p[2] = z2 * pow_pair<BITS, J, 2>(1.0f / kMul);
-        az.p[3] = z2 * pow_pair<BITS, J, 3>(1.0f / kMul);
-        d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(az.h, b.h, d[rr], 0, 0, 0);
+    for (int j = 0; j < 4; j++) b[j].v = *reinterpret_cast<const uint4*>(xb + tl * 128 + j * 32);
+    if constexpr (GROUP == 128) {
+      float4v t = MATGPTQ_MFMA(bias_operand(J0{}), b[0], zero4);
+      t = MATGPTQ_MFMA(bias_operand(J1{}), b[1], t);
+      t = MATGPTQ_MFMA(bias_operand(J2{}), b[2], t);
+      t = MATGPTQ_MFMA(bias_operand(J3{}), b[3], t);
+#pragma unroll
+      for (int rr = 0; rr < R; rr++) {
+        float4v v = MATGPTQ_MFMA(raw_operand(st, u, rr, J0{}), b[0], t);
+        v = MATGPTQ_MFMA(raw_operand(st, u, rr, J1{}), b[1], v);
+        v = MATGPTQ_MFMA(raw_operand(st, u, rr, J2{}), b[2], v);
+        v = MATGPTQ_MFMA(raw_operand(st, u, rr, J3{}), b[3], v);
+        if constexpr (ZP) {
+          const _Float16 zv = st.z[u][rr][0];
+          v = MATGPTQ_MFMA(zero_operand(zv, J0{}), b[0], v);
+          v = MATGPTQ_MFMA(zero_operand(zv, J1{}), b[1], v);
+          v = MATGPTQ_MFMA(zero_operand(zv, J2{}), b[2], v);
+          v = MATGPTQ_MFMA(zero_operand(zv, J3{}), b[3], v);
+        }
+        fold(st.s[u][rr][0], rr, v);
       }
-      if constexpr (GROUP == 32) fold_group(st.s[u][rr][J], rr);
+    } else if constexpr (GROUP == 32) {
+      auto octet = [&](auto jtag) {
+        constexpr int J = decltype(jtag)::value;
+        const float4v t = MATGPTQ_MFMA(bias_operand(jtag), b[J], zero4);
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) {
+          float4v v = MATGPTQ_MFMA(raw_operand(st, u, rr, jtag), b[J], t);
+          if constexpr (ZP) v = MATGPTQ_MFMA(zero_operand(st.z[u][rr][J], jtag), b[J], v);
+          fold(st.s[u][rr][J], rr, v);
+        }
+      };
+      octet(J0{});
+      octet(J1{});
+      octet(J2{});
+      octet(J3{});
+    } else {
+      db = MATGPTQ_MFMA(bias_operand(J0{}), b[0], db);
+      db = MATGPTQ_MFMA(bias_operand(J1{}), b[1], db);
+      db = MATGPTQ_MFMA(bias_operand(J2{}), b[2], db);
+      db = MATGPTQ_MFMA(bias_operand(J3{}), b[3], db);
+#pragma unroll
+      for (int rr = 0; rr < R; rr++) {
+        d[rr] = MATGPTQ_MFMA(raw_operand(st, u, rr, J0{}), b[0], d[rr]);
+        d[rr] = MATGPTQ_MFMA(raw_operand(st, u, rr, J1{}), b[1], d[rr]);
+        d[rr] = MATGPTQ_MFMA(raw_operand(st, u, rr, J2{}), b[2], d[rr]);
+        d[rr] = MATGPTQ_MFMA(raw_operand(st, u, rr, J3{}), b[3], d[rr]);
+        if constexpr (ZP) {
+          d[rr] = MATGPTQ_MFMA(zero_operand(zrow[rr], J0{}), b[0], d[rr]);
+          d[rr] = MATGPTQ_MFMA(zero_operand(zrow[rr], J1{}), b[1], d[rr]);
+          d[rr] = MATGPTQ_MFMA(zero_operand(zrow[rr], J2{}), b[2], d[rr]);
+          d[rr] = MATGPTQ_MFMA(zero_operand(zrow[rr], J3{}), b[3], d[rr]);
+        }
+      }
     }
   };
+#undef MATGPTQ_MFMA
 
   auto compute_stage = [&](const StageT& st, int c0, int c1, int stage) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int t = c0 + ws + W * (stage * U + u);
-      if (t < c1) {
-        const int tl = t - c0;
-        octet_step(st, u, tl, std::integral_constant<int, 0>{});
-        octet_step(st, u, tl, std::integral_constant<int, 1>{});
-        octet_step(st, u, tl, std::integral_constant<int, 2>{});
-        octet_step(st, u, tl, std::integral_constant<int, 3>{});
-        if constexpr (GROUP == 128) {
-#pragma unroll
-          for (int rr = 0; rr < R; rr++) fold_group(st.s[u][rr][0], rr);
-        }
-      }
+      if (t < c1) tile_step(st, u, t - c0);
     }
   };
 
-  auto stages_of = [&](int c0, int c1, bool live) {
+  auto stages_of = [&](int c0, int c1) {
     const int span = c1 - c0 - ws;  // this wave owns tiles c0+ws, c0+ws+W, ... below c1
     const int my_tiles = (live && span > 0) ? (span + W - 1) / W : 0;
     return (my_tiles + U - 1) / U;
   };
 
-  int it = blockIdx.x;
-  bool have_first = false;  // stage 0 of the coming group is already in `cur`
-  if (single) {
-    const int rb0 = (it * S + slot) * R;
-    if (it < sh.n_groups && rb0 < a.row_blocks && ws < a.k_tiles) {
-      load_stage(cur, rb0, 0, a.k_tiles, 0);  // weights first: they have the longest way to come
-      have_first = true;
+  auto run_stages = [&](int c0, int c1, int n_stages) {
+    if constexpr (STREAM) {
+      // two stages per trip so that the prefetched stage needs no register copy
+      for (int stage = 0; stage < n_stages; stage += 2) {
+        if (stage + 1 < n_stages) load_stage(nxt, c0, c1, stage + 1);
+        compute_stage(cur, c0, c1, stage);
+        if (stage + 1 < n_stages) {
+          if (stage + 2 < n_stages) load_stage(cur, c0, c1, stage + 2);
+          compute_stage(nxt, c0, c1, stage + 1);
+        }
+      }
+    } else {
+      for (int stage = 0; stage < n_stages; stage++) {
+        if (stage > 0) load_stage(cur, c0, c1, stage);
+        compute_stage(cur, c0, c1, stage);
+      }
     }
+  };
+
+  if constexpr (!CHUNKED) {
+    // all of X' fits in LDS: weights first (they have the longest way to come), then X'
+    const int n_stages = stages_of(0, a.k_tiles);
+    if (n_stages > 0) load_stage(cur, 0, a.k_tiles, 0);
 #ifndef MATGPTQ_DEBUG_NOSTAGE
     stage_x(0, a.k_tiles);
     __syncthreads();
 #endif
-  }
-
-  for (; it < sh.n_groups; it += gridDim.x) {
-    const int rb_wg = it * S * R;          // first row block of the group
-    const int rb0 = rb_wg + slot * R;      // first row block of this wave
-    const bool live = rb0 < a.row_blocks;  // the last group may have idle slots
-#pragma unroll
-    for (int rr = 0; rr < R; rr++) {
-      acc[rr] = float4v{0.f, 0.f, 0.f, 0.f};
-      d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
-    }
-    if constexpr (!GROUPED && ZP) {
-      if (live) {
-#pragma unroll
-        for (int rr = 0; rr < R; rr++)
-        {
-          const _Float16 zv = reinterpret_cast<const _Float16*>(a.zeros)[(size_t)(rb0 + rr) * 16 + r16];
-          cur.z[0][rr][0] = zv;
-          if constexpr (STREAM) nxt.z[0][rr][0] = zv;
-        }
-      }
-    }
-
-    // K is walked in chunks of kc tiles so that the LDS copy of X' stays small.
+    run_stages(0, a.k_tiles, n_stages);
+  } else {
+    // K is walked in chunks of kc tiles so that the LDS copy of X' stays small
     for (int c0 = 0; c0 < a.k_tiles; c0 += kc) {
       const int c1 = c0 + kc < a.k_tiles ? c0 + kc : a.k_tiles;
-      const int n_stages = stages_of(c0, c1, live);
-      if (!have_first && n_stages > 0) load_stage(cur, rb0, c0, c1, 0);
-      have_first = false;
-      if (!single) {
-        __syncthreads();  // all waves are done with the previous contents of X'
-        stage_x(c0, c1);
-        __syncthreads();
-      }
-
-      // next group's first stage, issued as soon as a register buffer is free
-      const int it_next = it + (int)gridDim.x;
-      auto prefetch_next = [&]() {
-        if (single && it_next < sh.n_groups) {
-          const int rbn = (it_next * S + slot) * R;
-          if (rbn < a.row_blocks && ws < a.k_tiles) {
-            load_stage(cur, rbn, 0, a.k_tiles, 0);
-            have_first = true;
-          }
-        }
-      };
-
-      if constexpr (STREAM) {
-        // two stages per trip so that the prefetched stage needs no register copy
-        for (int stage = 0; stage < n_stages; stage += 2) {
-          if (stage + 1 < n_stages) load_stage(nxt, rb0, c0, c1, stage + 1);
-          compute_stage(cur, c0, c1, stage);
-          if (stage + 1 < n_stages) {
-            if (stage + 2 < n_stages) load_stage(cur, rb0, c0, c1, stage + 2);
-            else prefetch_next();
-            compute_stage(nxt, c0, c1, stage + 1);
-          } else {
-            prefetch_next();
-          }
-        }
-        if (n_stages == 0) prefetch_next();
-      } else {
-        for (int stage = 0; stage < n_stages; stage++) {
-          if (stage > 0) load_stage(cur, rb0, c0, c1, stage);
-          compute_stage(cur, c0, c1, stage);
-        }
-        prefetch_next();
-      }
+      const int n_stages = stages_of(c0, c1);
+      if (n_stages > 0) load_stage(cur, c0, c1, 0);
+      if (c0 > 0) __syncthreads();  // all waves are done with the previous contents of X'
+      stage_x(c0, c1);
+      __syncthreads();
+      run_stages(c0, c1, n_stages);
     }
+  }
 
-    if constexpr (!GROUPED) {
-      if (live) {
+  if constexpr (!GROUPED) {
+    if (live) {
 #pragma unroll
-        for (int rr = 0; rr < R; rr++)
-          fold_group(*reinterpret_cast<const uint2*>(a.scales + (size_t)(rb0 + rr) * 16 + 4 * q), rr);
-      }
+      for (int rr = 0; rr < R; rr++)
+        fold(*reinterpret_cast<const uint2*>(a.scales + (size_t)(rb0 + rr) * 16 + 4 * q), rr, d[rr] + db);
     }
+  }
 
 #ifdef MATGPTQ_DEBUG_NOREDUCE
-    if (acc[0][0] == 1.2345f) a.y[tid] = 1;
-    continue;
+  if (acc[0][0] == 1.2345f) a.y[tid] = 1;
+  return;
 #endif
-    // combine the W partial sums of each slot: red[wave][rr][lane*4 + i]
-    if (it != (int)blockIdx.x) __syncthreads();  // the previous group's sums have been read
+  // combine the W partial sums of each slot: red[wave][rr][lane*4 + i]
 #pragma unroll
-    for (int rr = 0; rr < R; rr++)
-      *reinterpret_cast<float4v*>(red + ((wave * R + rr) * 64 + lane) * 4) = acc[rr];
-    __syncthreads();
+  for (int rr = 0; rr < R; rr++)
+    *reinterpret_cast<float4v*>(red + ((wave * R + rr) * 64 + lane) * 4) = acc[rr];
+  __syncthreads();
 
-    const int outs = a.M << sh.lg_rows;
-    for (int o = tid; o < outs; o += blockDim.x) {
-      const int n = o >> sh.lg_rows;
-      const int rowl = o & ((1 << sh.lg_rows) - 1);
-      const int rbl = rowl >> 4, row = rowl & 15;  // row block inside the group
-      const int sl = rbl / R, rr = rbl % R;
-      const int grow = (rb_wg + rbl) * 16 + row;
-      if (grow < a.N) {
-        const float* src = red + ((sl * W) * R + rr) * 256 + (((row >> 2) * 16 + n) << 2) + (row & 3);
-        float sum = 0.f;
-        for (int w = 0; w < W; w++) sum += src[w * R * 256];
-        reinterpret_cast<_Float16*>(a.y)[(size_t)n * a.N + grow] = (_Float16)(sum * kMul);
-      }
+  const int outs = a.M << sh.lg_rows;
+  for (int o = tid; o < outs; o += blockDim.x) {
+    const int n = o >> sh.lg_rows;
+    const int rowl = o & ((1 << sh.lg_rows) - 1);
+    const int rbl = rowl >> 4, row = rowl & 15;  // row block inside the workgroup
+    const int sl = rbl / R, rr = rbl % R;
+    const int grow = (rb_wg + rbl) * 16 + row;
+    if (grow < a.N) {
+      const float* src = red + ((sl * W) * R + rr) * 256 + (((row >> 2) * 16 + n) << 2) + (row & 3);
+      float sum = 0.f;
+      for (int w = 0; w < W; w++) sum += src[w * R * 256];
+      reinterpret_cast<_Float16*>(a.y)[(size_t)n * a.N + grow] = (_Float16)(sum * kMul);
     }
   }
 }
@@ -361,26 +385,34 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
 template <int BITS, int GROUP, bool ZP, int R>
 __global__ void __launch_bounds__(1024)
 decode_stream_kernel(const GemmArgs a, const DecodeShape sh) {
-  decode_body<BITS, GROUP, ZP, R, true>(a, sh);
+  decode_body<BITS, GROUP, ZP, R, true, false>(a, sh);
 }
 
 // burst: up to 8 waves per workgroup, register budget for 6 waves per SIMD
 template <int BITS, int GROUP, bool ZP, int R>
 __global__ void __launch_bounds__(512, 6)
 decode_burst_kernel(const GemmArgs a, const DecodeShape sh) {
-  decode_body<BITS, GROUP, ZP, R, false>(a, sh);
+  decode_body<BITS, GROUP, ZP, R, false, false>(a, sh);
+}
+
+// chunked: X' staged kc tiles at a time (large M * K)
+template <int BITS, int GROUP, bool ZP, int R>
+__global__ void __launch_bounds__(512, 4)
+decode_chunked_kernel(const GemmArgs a, const DecodeShape sh) {
+  decode_body<BITS, GROUP, ZP, R, false, true>(a, sh);
 }
 
 template <int GROUP, bool ZP, int R>
-hipError_t launch_one(const GemmArgs& a, int S, int W, int kc, int max_wgs, bool stream_flavour,
-                      size_t smem, hipStream_t stream) {
+hipError_t launch_one(const GemmArgs& a, int S, int W, int kc, bool stream_flavour, size_t smem,
+                      hipStream_t stream) {
   const int per_wg = S * R;
-  const int n_groups = (a.row_blocks + per_wg - 1) / per_wg;
   int lg = 4;
   while ((1 << lg) < per_wg * 16) lg++;
-  const dim3 grid(max_wgs > 0 && max_wgs < n_groups ? max_wgs : n_groups), block(64 * S * W);
-  const DecodeShape sh{S, W, kc, n_groups, lg};
-  if (stream_flavour)
+  const dim3 grid((a.row_blocks + per_wg - 1) / per_wg), block(64 * S * W);
+  const DecodeShape sh{S, W, kc, lg};
+  if (kc < a.k_tiles)
+    hipLaunchKernelGGL((decode_chunked_kernel<kBits, GROUP, ZP, R>), grid, block, smem, stream, a, sh);
+  else if (stream_flavour)
     hipLaunchKernelGGL((decode_stream_kernel<kBits, GROUP, ZP, R>), grid, block, smem, stream, a, sh);
   else
     hipLaunchKernelGGL((decode_burst_kernel<kBits, GROUP, ZP, R>), grid, block, smem, stream, a, sh);
@@ -388,11 +420,11 @@ hipError_t launch_one(const GemmArgs& a, int S, int W, int kc, int max_wgs, bool
 }
 
 template <int GROUP, bool ZP>
-hipError_t launch_r(const GemmArgs& a, int R, int S, int W, int kc, int max_wgs, bool sf,
-                    size_t smem, hipStream_t s) {
-  if (R == 1) return launch_one<GROUP, ZP, 1>(a, S, W, kc, max_wgs, sf, smem, s);
-  if (R == 2) return launch_one<GROUP, ZP, 2>(a, S, W, kc, max_wgs, sf, smem, s);
-  return launch_one<GROUP, ZP, 4>(a, S, W, kc, max_wgs, sf, smem, s);
+hipError_t launch_r(const GemmArgs& a, int R, int S, int W, int kc, bool sf, size_t smem,
+                    hipStream_t s) {
+  if (R == 1) return launch_one<GROUP, ZP, 1>(a, S, W, kc, sf, smem, s);
+  if (R == 2) return launch_one<GROUP, ZP, 2>(a, S, W, kc, sf, smem, s);
+  return launch_one<GROUP, ZP, 4>(a, S, W, kc, sf, smem, s);
 }
 
 }  // namespace
@@ -400,23 +432,22 @@ hipError_t launch_r(const GemmArgs& a, int R, int S, int W, int kc, int max_wgs,
 // Entry of this translation unit: launch the decode kernel for bitwidth MATGPTQ_BITS.
 // R in {1,2,4} row blocks per wave, S slots and W k-slices per workgroup
 // (S*W <= 16 for the stream flavour, <= 8 for burst), kc = tiles of K staged in LDS at
-// a time, max_wgs = cap on the grid (0 = one workgroup per group of row blocks; otherwise
-// workgroups walk several groups), smem = dynamic LDS bytes (see decode_lds_bytes in abi.hip).
+// a time (kc < K/128 selects the chunked kernel, 8 waves at most), smem = dynamic LDS
+// bytes (see decode_lds_bytes in abi.hip).
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 hipError_t MATGPTQ_CAT(launch_decode_b, MATGPTQ_BITS)(const GemmArgs& a, int group_size, int R,
-                                                      int S, int W, int kc, int max_wgs,
-                                                      bool stream_flavour, size_t smem,
-                                                      hipStream_t stream) {
+                                                      int S, int W, int kc, bool stream_flavour,
+                                                      size_t smem, hipStream_t stream) {
   const bool zp = a.zeros != nullptr;
   if (group_size == 128)
-    return zp ? launch_r<128, true>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream)
-              : launch_r<128, false>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream);
+    return zp ? launch_r<128, true>(a, R, S, W, kc, stream_flavour, smem, stream)
+              : launch_r<128, false>(a, R, S, W, kc, stream_flavour, smem, stream);
   if (group_size == 32)
-    return zp ? launch_r<32, true>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream)
-              : launch_r<32, false>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream);
-  return zp ? launch_r<-1, true>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream)
-            : launch_r<-1, false>(a, R, S, W, kc, max_wgs, stream_flavour, smem, stream);
+    return zp ? launch_r<32, true>(a, R, S, W, kc, stream_flavour, smem, stream)
+              : launch_r<32, false>(a, R, S, W, kc, stream_flavour, smem, stream);
+  return zp ? launch_r<-1, true>(a, R, S, W, kc, stream_flavour, smem, stream)
+            : launch_r<-1, false>(a, R, S, W, kc, stream_flavour, smem, stream);
 }
 
 }  // namespace matgptq

@@ -109,17 +109,12 @@ def test_prefill_every_tile_configuration(cfg):
 
 
 def _decode_variants():
-    out = []
-    for v in range(1, 43):
-        for flavour in (1, 2):
-            for cap in (1, 2):
-                out.append(1 | (v << 8) | (flavour << 16) | (cap << 18))
-    return out
+    return [1 | (v << 8) | (flavour << 16) for v in range(1, 43) for flavour in (1, 2)]
 
 
 def test_decode_every_work_split():
-    # all (R, S, W) shapes, both flavours, capped (persistent) and uncapped grids; 65 row
-    # blocks leave idle slots in the last group, K = 4096 gives up to 32 tiles per wave
+    # all (R, S, W) shapes in both flavours; 65 row blocks leave idle slots in the last
+    # workgroup, K = 4096 gives up to 32 tiles per wave
     lay = G.Layer(1040, 4096, 4, 128, seed=4)
     x = o.make_activations(3, 4096, seed=2)
     ran = 0
@@ -131,7 +126,7 @@ def test_decode_every_work_split():
             continue
         G.assert_close_to_oracle(y, x, lay.w, f"flags {flags:#x}")
         ran += 1
-    assert ran >= 100
+    assert ran >= 60
 
 
 @pytest.mark.parametrize("b", (3, 4))
@@ -147,7 +142,7 @@ def test_chunked_activation_staging():
     # M = 16 with K = 14336 does not fit in LDS at once: the kernel walks K in chunks
     lay = G.Layer(64, 14336, 4, 128, seed=7)
     x = o.make_activations(16, 14336, seed=7)
-    assert "kc112" not in _lib.describe_plan(4, 128, 64, 14336, 16, True)
+    assert _lib.describe_plan(4, 128, 64, 14336, 16, True).startswith("decode-chunked")
     G.assert_close_to_oracle(lay.run(x), x, lay.w, "chunked")
 
 
