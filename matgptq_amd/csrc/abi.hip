@@ -82,7 +82,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   }
   if (variant != 0) {
     if (variant >= 64) {
-      if (variant - 64 > 4) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 7) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->cfg = variant - 64;
     } else {

@@ -172,10 +172,12 @@ __device__ __forceinline__ BufRsrc make_rsrc(const void* p, uint32_t bytes) {
 }
 
 // Loads the BITS words of `lane` from the tile that starts `tile_bytes` into the buffer
-// (wave-uniform), one load per segment, as streaming reads.
-template <int BITS>
+// (wave-uniform), one load per segment.  AUX = kAuxStream for data read once (decode),
+// 0 for data other workgroups read again (prefill).
+template <int BITS, int AUX = kAuxStream>
 __device__ __forceinline__ void load_tile_words(BufRsrc rs, uint32_t tile_bytes, int lane,
                                                 uint32_t (&w)[BITS]) {
+  constexpr int kAuxStream = AUX;  // shadows the global constant below on purpose
   if constexpr (BITS == 2) {
     const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane * 8, tile_bytes, kAuxStream);
     w[0] = v.x; w[1] = v.y;

@@ -58,8 +58,11 @@ __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const U
   a.p[3] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 3), ZP>(raw[3], zrel, scale);
 }
 
+// two waves per SIMD whenever the accumulators leave room for it
+constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 <= 128 ? 2 : 1; }
+
 template <int BITS, int GROUP, bool ZP, int RBW, int MT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, prefill_min_waves(RBW, MT))
 prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   constexpr int TM = 16 * MT;
   constexpr int GPT = GROUP == 32 ? 4 : 1;
@@ -69,7 +72,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile offsets stay scalar
   const int r16 = lane & 15;
   const int q = lane >> 4;
 
@@ -85,6 +88,9 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
   const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
   const BufRsrc wres = make_rsrc(a.packed, (uint32_t)a.row_blocks * rb_bytes);
+  const uint32_t aux_bytes = (uint32_t)a.row_blocks * a.G * 32;  // scales / zeros: [N/16][G][16] halves
+  const BufRsrc sres = make_rsrc(a.scales, aux_bytes);
+  const BufRsrc zres = make_rsrc(ZP ? a.zeros : a.scales, aux_bytes);
 
   float4v acc[RBW][MT];
 #pragma unroll
@@ -102,14 +108,20 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
       const int rb = rb_first + rr;
+#ifdef MATGPTQ_DEBUG_NOWLOAD
+      if (rb < a.row_blocks && kb == 0) {
+#else
       if (rb < a.row_blocks) {
-        load_tile_words<BITS>(wres, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
+#endif
+        load_tile_words<BITS, 0>(wres, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
 #pragma unroll
         for (int gg = 0; gg < GPT; gg++) {
-          const size_t g = GROUP == -1 ? 0 : (size_t)kb * GPT + gg;
-          const size_t so = ((size_t)rb * a.G + g) * 16 + r16;
-          s[rr][gg] = reinterpret_cast<const _Float16*>(a.scales)[so];
-          if constexpr (ZP) z[rr][gg] = reinterpret_cast<const _Float16*>(a.zeros)[so] - (_Float16)128.0f;
+          const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
+          const uint32_t so = ((uint32_t)rb * a.G + g) * 32;  // bytes
+          s[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(sres, r16 * 2, so, 0));
+          if constexpr (ZP)
+            z[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(zres, r16 * 2, so, 0)) -
+                        (_Float16)128.0f;
         }
       } else {
 #pragma unroll
@@ -128,7 +140,11 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
       const int row = chunk >> 3, col8 = chunk & 7;
       const int m = m0 + row;
       xreg[c] = make_uint4(0u, 0u, 0u, 0u);
+#ifdef MATGPTQ_DEBUG_NOXLOAD
+      if (m < -1)
+#else
       if (m < a.M)
+#endif
         xreg[c] = *reinterpret_cast<const uint4*>(a.x + (size_t)m * a.K + (size_t)h * kXs + col8 * 8);
     }
   };
@@ -141,34 +157,48 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     }
   };
 
-  // half step: octets J0, J0+1 of the current tile against LDS buffer `buf`
+  // half step: octets J0, J0+1 of the current tile against LDS buffer `buf`.  All operand
+  // reads of a 32-column step are issued before its first MFMA, so that LDS latency is
+  // paid once per step and not once per activation tile.
   auto half_step = [&](int buf, auto j0tag) {
     constexpr int J0 = decltype(j0tag)::value;
-#pragma unroll
-    for (int jj = 0; jj < 2; jj++) {
+    auto k32 = [&](auto jtag) {
+      constexpr int J = decltype(jtag)::value;
+      constexpr int jj = J - J0;
       Frag aw[RBW];
 #pragma unroll
       for (int rr = 0; rr < RBW; rr++) {
-        const int gg = GROUP == 32 ? (J0 + jj) : 0;
+        const int gg = GROUP == 32 ? J : 0;
         _Float16 s1 = scur[rr][gg];
         if constexpr (!ZP) s1 = (_Float16)((float)s1 * (float)(1 << (8 - BITS)));
         const half2v sc = {s1, s1};
         half2v zr = {(_Float16)0.f, (_Float16)0.f};
         if constexpr (ZP) zr = half2v{zcur[rr][gg], zcur[rr][gg]};
-        if (jj == 0)
-          dequant_octet<BITS, J0, ZP>(wcur[rr], kc_unpack, zr, sc, aw[rr]);
-        else
-          dequant_octet<BITS, J0 + 1, ZP>(wcur[rr], kc_unpack, zr, sc, aw[rr]);
+#ifdef MATGPTQ_DEBUG_NODEQUANT
+        aw[rr].u[0] = wcur[rr][0]; aw[rr].u[1] = wcur[rr][1 % BITS]; aw[rr].u[2] = wcur[rr][0] ^ J; aw[rr].u[3] = wcur[rr][1 % BITS];
+        (void)sc; (void)zr;
+#else
+        dequant_octet<BITS, J, ZP>(wcur[rr], kc_unpack, zr, sc, aw[rr]);
+#endif
       }
+      // activation operands in groups of four tiles: their reads are in flight together
+      constexpr int MG = MT < 4 ? MT : 4;
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) {
-        Frag b;
-        b.v = *reinterpret_cast<const uint4*>(&xs[buf][(mt * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
+      for (int m0g = 0; m0g < MT; m0g += MG) {
+        Frag b[MG];
 #pragma unroll
-        for (int rr = 0; rr < RBW; rr++)
-          acc[rr][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b.h, acc[rr][mt], 0, 0, 0);
+        for (int i = 0; i < MG; i++)
+          b[i].v = *reinterpret_cast<const uint4*>(&xs[buf][((m0g + i) * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
+#pragma unroll
+        for (int i = 0; i < MG; i++) {
+#pragma unroll
+          for (int rr = 0; rr < RBW; rr++)
+            acc[rr][m0g + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b[i].h, acc[rr][m0g + i], 0, 0, 0);
+        }
       }
-    }
+    };
+    k32(std::integral_constant<int, J0>{});
+    k32(std::integral_constant<int, J0 + 1>{});
   };
 
   // prologue
@@ -236,7 +266,10 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 1: return launch_cfg<GROUP, ZP, 8, 8>(a, s);   // 128 x 512
     case 2: return launch_cfg<GROUP, ZP, 4, 4>(a, s);   // 64 x 256
     case 3: return launch_cfg<GROUP, ZP, 2, 8>(a, s);   // 128 x 128
-    default: return launch_cfg<GROUP, ZP, 2, 2>(a, s);  // 32 x 128
+    case 4: return launch_cfg<GROUP, ZP, 2, 2>(a, s);   // 32 x 128
+    case 5: return launch_cfg<GROUP, ZP, 8, 4>(a, s);   // 64 x 512
+    case 6: return launch_cfg<GROUP, ZP, 8, 2>(a, s);   // 32 x 512
+    default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 }
 

@@ -101,7 +101,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(5))
+@pytest.mark.parametrize("cfg", range(8))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
