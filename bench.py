@@ -36,6 +36,11 @@ LLAMA3_8B = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "
 LLAMA3_70B = {"qkv": (10240, 8192), "o": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
 GROUP = 128
 RING_BYTES = 2.5e9
+COUNTER_COPY_BYTES = 256 * 1024 * 1024
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --counter-pass`, each counter scaled by what it reads for the 256 MiB elementwise copy
+# of the same run.  Keyed by the kernel plan the figure was taken on: a different plan reports null.
+MEASURED_TRAFFIC = {}
 
 
 def algorithmic_bytes(n, k, m, bits, zero_points=True):
@@ -50,6 +55,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
+    ap.add_argument("--counter-pass", action="store_true",
+                    help="for rocprofv3 --pmc runs: launch only the dominant kernel over the ring of weight "
+                         "copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's yardstick)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -107,8 +115,28 @@ def main() -> int:
                 best = min(best, e0.elapsed_time(e1) * 1e-3)
         return best
 
-    # ------------------------------------------------------------------ headline
     bits = 4
+    if args.counter_pass:
+        n, k = LLAMA3_8B["gate_up"]
+        copies = int(RING_BYTES // (n * k * bits // 8)) + 1
+        ring = make_ring(n, k, bits, copies)
+        sc, zr = make_aux(n, k)
+        x = torch.randn(1, k, device=dev, generator=g).to(torch.float16)
+        y = torch.empty(1, n, dtype=torch.float16, device=dev)
+        with torch.cuda.stream(stream):
+            for i in range(2 * copies):
+                launch(bits, n, k, x, ring[i % copies], sc, zr, y)
+            stream.synchronize()
+            src = torch.zeros(COUNTER_COPY_BYTES // 4, dtype=torch.int32, device=dev)
+            dst = torch.empty_like(src)
+            for _ in range(4):
+                torch.add(src, 1, out=dst)  # one elementwise kernel: reads and writes COUNTER_COPY_BYTES
+            stream.synchronize()
+        print(json.dumps({"counter_pass": _lib.describe_plan(bits, GROUP, n, k, 1, True),
+                          "launches": 2 * copies, "copy_bytes_each_way": COUNTER_COPY_BYTES}))
+        return 0
+
+    # ------------------------------------------------------------------ headline
     step_bytes = sum(n * k * bits // 8 for n, k in LLAMA3_8B.values())
     copies = max(2, int(RING_BYTES // step_bytes) + 1)
     rings = {name: make_ring(n, k, bits, copies) for name, (n, k) in LLAMA3_8B.items()}
@@ -146,7 +174,7 @@ def main() -> int:
         "peak": HBM_PEAK_GBPS,
         "unit": "GB/s",
         "frac": round(dom_bytes / t_dom / 1e9 / HBM_PEAK_GBPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC.get(_lib.describe_plan(bits, GROUP, n, k, 1, True)),
         "us_per_launch": round(t_dom * 1e6, 2),
         "algorithmic_bytes": dom_bytes,
     }

@@ -73,7 +73,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   // row blocks to keep every CU busy that way
   int W = 8, S = 1;
   while (W > 1 && W > k_tiles) { W >>= 1; S <<= 1; }
-  int R = row_blocks >= 1024 ? 4 : 1;
+  // (group 32 carries four scales and zeros per tile and row block: two row blocks at most)
+  int R = row_blocks >= 1024 ? (group_size == 32 ? 2 : 4) : 1;
   // default prefill tile
   if (!p->decode) {
     if (M <= 32) p->cfg = 4;
@@ -122,7 +123,6 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   p->smem = decode_lds_bytes(R, S, W, (int)kc, M);
   if (kc < k_tiles && S * W > 8) return variant != 0 ? MATGPTQ_EVARIANT : MATGPTQ_ESIZE;
   (void)zp;
-  (void)group_size;
   (void)bits;
   return MATGPTQ_OK;
 }

@@ -37,9 +37,11 @@ namespace {
 constexpr int kBits = MATGPTQ_BITS;
 
 // Tiles a wave loads per pipeline stage, for R row blocks per wave.
-constexpr int tiles_in_flight(int bits, int r) {
+// Group 32 carries four scales (and zeros) per tile and row block, so fewer tiles fit.
+constexpr int tiles_in_flight(int bits, int r, int group = 128) {
   const int u = (16 + r * bits - 1) / (r * bits);
-  return u < 1 ? 1 : (u > 4 ? 4 : u);
+  const int cap = group == 32 ? (r >= 4 ? 1 : 2) : 4;
+  return u < 1 ? 1 : (u > cap ? cap : u);
 }
 
 // fp16 pair constant for pair i of octet J: 2^p in both halves, times `f`.
@@ -69,7 +71,7 @@ struct Stage {
 // STREAM: double-buffered stages.  CHUNKED: X' is staged kc tiles at a time.
 template <int BITS, int GROUP, bool ZP, int R, bool STREAM, bool CHUNKED>
 __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape sh) {
-  constexpr int U = tiles_in_flight(BITS, R);
+  constexpr int U = tiles_in_flight(BITS, R, GROUP);
   constexpr bool GROUPED = GROUP != -1;
   constexpr int GPT = GROUP == 32 ? 4 : 1;  // groups per tile
   constexpr float kMul = (float)(1 << (8 - BITS));
@@ -98,67 +100,112 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
   constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
   const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
   const uint32_t aux_bytes = (uint32_t)a.row_blocks * a.G * 32;  // scales / zeros: [N/16][G][16] halves
-  const BufRsrc wres = make_rsrc(a.packed, (uint32_t)a.row_blocks * rb_bytes);
-  const BufRsrc sres = make_rsrc(a.scales, aux_bytes);
-  const BufRsrc zres = make_rsrc(ZP ? a.zeros : a.scales, aux_bytes);
+  const uint32_t w_bytes = (uint32_t)a.row_blocks * rb_bytes;
 
   using StageT = Stage<BITS, R, U, GPT, ZP>;
   StageT cur, nxt;
   const UnpackConsts<BITS> kc_unpack;
 
-  // loads stage `stage` of chunk [c0, c1): tiles c0 + ws + W * (stage * U + u)
+  // loads stage `stage` of chunk [c0, c1): tiles c0 + ws + W * (stage * U + u).  Branch-free:
+  // a tile beyond the chunk is read through a descriptor of zero length (every lane out of
+  // range, nothing fetched), so that the count of loads in flight is known at compile time
+  // and later waits can be exact.
   auto load_stage = [&](StageT& st, int c0, int c1, int stage) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int t = c0 + ws + W * (stage * U + u);
-      if (t < c1) {
+      const bool valid = live && t < c1;
+      const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
+      const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
+      const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
 #pragma unroll
-        for (int rr = 0; rr < R; rr++) {
-          load_tile_words<BITS>(wres, (uint32_t)(rb0 + rr) * rb_bytes + (uint32_t)t * tile_bytes, lane,
-                                st.w[u][rr]);
-          if constexpr (GROUPED) {
+      for (int rr = 0; rr < R; rr++) {
+        load_tile_words<BITS>(wr, (uint32_t)(rb0 + rr) * rb_bytes + (uint32_t)t * tile_bytes, lane,
+                              st.w[u][rr]);
+        if constexpr (GROUPED) {
 #pragma unroll
-            for (int gg = 0; gg < GPT; gg++) {
-              const uint32_t so = ((uint32_t)(rb0 + rr) * a.G + (uint32_t)t * GPT + gg) * 32;  // bytes
-              const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(sres, q * 8, so, 0);
-              st.s[u][rr][gg] = make_uint2(sv.x, sv.y);
-              if constexpr (ZP) {
-                const uint16_t zv = __builtin_amdgcn_raw_buffer_load_b16(zres, r16 * 2, so, 0);
-                st.z[u][rr][gg] = __builtin_bit_cast(_Float16, zv);
-              }
+          for (int gg = 0; gg < GPT; gg++) {
+            const uint32_t so = ((uint32_t)(rb0 + rr) * a.G + (uint32_t)t * GPT + gg) * 32;  // bytes
+            const u32x2 sv = __builtin_amdgcn_raw_buffer_load_b64(sr, q * 8, so, 0);
+            st.s[u][rr][gg] = make_uint2(sv.x, sv.y);
+            if constexpr (ZP) {
+              const uint16_t zv = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
+              st.z[u][rr][gg] = __builtin_bit_cast(_Float16, zv);
             }
           }
         }
       }
     }
+    // all loads of a stage are issued before anything that uses them
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  // X' = X * 2^-p for columns [c0*128, c1*128).  A thread moves eight consecutive k
-  // (one octet of one k-quarter); p depends on the pair inside the octet and, for
-  // b = 2, on the parity of the octet index (k / 32) % 4.
-  auto stage_x = [&](int c0, int c1) {
-    const int chunks = (c1 - c0) * 16;
-    for (int m = 0; m < a.M; m++) {
-      const uint4* src = reinterpret_cast<const uint4*>(a.x + (size_t)m * a.K + (size_t)c0 * 128);
-      for (int c = tid; c < chunks; c += blockDim.x) {
-        Frag v;
-        v.v = src[c];
-        if constexpr (BITS != 8) {
-          const bool odd = BITS == 2 && ((c >> 2) & 1) != 0;  // octet index k/32 = c/4
-          if (odd) {
-            v.p[0] = v.p[0] * inv_pow_pair<BITS, 1, 0>();
-            v.p[1] = v.p[1] * inv_pow_pair<BITS, 1, 1>();
-            v.p[2] = v.p[2] * inv_pow_pair<BITS, 1, 2>();
-            v.p[3] = v.p[3] * inv_pow_pair<BITS, 1, 3>();
-          } else {
-            v.p[0] = v.p[0] * inv_pow_pair<BITS, 0, 0>();
-            v.p[1] = v.p[1] * inv_pow_pair<BITS, 0, 1>();
-            v.p[2] = v.p[2] * inv_pow_pair<BITS, 0, 2>();
-            v.p[3] = v.p[3] * inv_pow_pair<BITS, 0, 3>();
-          }
-        }
-        *reinterpret_cast<uint4*>(xs + m * pitch + c * 8) = v.v;
+  auto scale_x = [&](half8& hv, bool odd) {
+    if constexpr (BITS != 8) {
+      Frag v;
+      v.h = hv;
+      if (odd) {
+        v.p[0] = v.p[0] * inv_pow_pair<BITS, 1, 0>();
+        v.p[1] = v.p[1] * inv_pow_pair<BITS, 1, 1>();
+        v.p[2] = v.p[2] * inv_pow_pair<BITS, 1, 2>();
+        v.p[3] = v.p[3] * inv_pow_pair<BITS, 1, 3>();
+      } else {
+        v.p[0] = v.p[0] * inv_pow_pair<BITS, 0, 0>();
+        v.p[1] = v.p[1] * inv_pow_pair<BITS, 0, 1>();
+        v.p[2] = v.p[2] * inv_pow_pair<BITS, 0, 2>();
+        v.p[3] = v.p[3] * inv_pow_pair<BITS, 0, 3>();
       }
+      hv = v.h;
+    }
+  };
+  // The copy of X' is latency-bound: a thread keeps XU loads in flight, and the first trip
+  // is issued BEFORE the weight loads of the first stage (memory returns in order, so an
+  // activation load queued behind them would not be usable until all of them had landed).
+  constexpr int XU = 4;
+  struct XTrip {
+    half8 v[XU];
+    int dst[XU];   // halves into xs
+    bool odd[XU];  // b = 2: parity of the octet index k/32 selects the shift set
+  };
+  auto x_fetch = [&](XTrip& t, int c0, int chunks, int base) {
+    const half8* src = reinterpret_cast<const half8*>(a.x + (size_t)c0 * 128);
+    const int total = a.M * chunks;
+    int off[XU];
+#pragma unroll
+    for (int i = 0; i < XU; i++) {
+      const int idx = base + i * (int)blockDim.x;
+      // Past the end a thread repeats the last chunk (same value to the same place): loads and
+      // stores stay unconditional, so none of them can be moved behind the weight loads.
+      const int cl = idx < total ? idx : total - 1;
+      int m = 0, c = cl;
+      if (a.M > 1) {
+        m = cl / chunks;
+        c = cl - m * chunks;
+      }
+      off[i] = m * (a.K / 8) + c;
+      t.dst[i] = m * pitch + c * 8;
+      t.odd[i] = BITS == 2 && ((c >> 2) & 1) != 0;  // octet index k/32 = c/4
+    }
+    // straight-line loads: the compiler can then wait for exactly these and no later load
+#pragma unroll
+    for (int i = 0; i < XU; i++) t.v[i] = src[off[i]];
+  };
+  auto x_commit = [&](XTrip& t) {
+#pragma unroll
+    for (int i = 0; i < XU; i++) {
+      scale_x(t.v[i], t.odd[i]);
+      *reinterpret_cast<half8*>(xs + t.dst[i]) = t.v[i];
+    }
+  };
+  // stores the prefetched first trip `t`, then copies the rest of columns [c0*128, c1*128)
+  auto stage_x = [&](XTrip& t, int c0, int c1) {
+    const int chunks = (c1 - c0) * 16;
+    const int total = a.M * chunks;
+    const int step = XU * (int)blockDim.x;
+    x_commit(t);
+    for (int base = tid + step; base < total; base += step) {
+      x_fetch(t, c0, chunks, base);
+      x_commit(t);
     }
   };
 
@@ -325,12 +372,16 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
     }
   };
 
+  XTrip xt;
   if constexpr (!CHUNKED) {
-    // all of X' fits in LDS: weights first (they have the longest way to come), then X'
+    // all of X' fits in LDS
     const int n_stages = stages_of(0, a.k_tiles);
-    if (n_stages > 0) load_stage(cur, 0, a.k_tiles, 0);
 #ifndef MATGPTQ_DEBUG_NOSTAGE
-    stage_x(0, a.k_tiles);
+    x_fetch(xt, 0, a.k_tiles * 16, tid);
+#endif
+    load_stage(cur, 0, a.k_tiles, 0);
+#ifndef MATGPTQ_DEBUG_NOSTAGE
+    stage_x(xt, 0, a.k_tiles);
     __syncthreads();
 #endif
     run_stages(0, a.k_tiles, n_stages);
@@ -339,9 +390,10 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
     for (int c0 = 0; c0 < a.k_tiles; c0 += kc) {
       const int c1 = c0 + kc < a.k_tiles ? c0 + kc : a.k_tiles;
       const int n_stages = stages_of(c0, c1);
-      if (n_stages > 0) load_stage(cur, c0, c1, 0);
+      x_fetch(xt, c0, (c1 - c0) * 16, tid);
+      load_stage(cur, c0, c1, 0);
       if (c0 > 0) __syncthreads();  // all waves are done with the previous contents of X'
-      stage_x(c0, c1);
+      stage_x(xt, c0, c1);
       __syncthreads();
       run_stages(c0, c1, n_stages);
     }
@@ -388,9 +440,10 @@ decode_stream_kernel(const GemmArgs a, const DecodeShape sh) {
   decode_body<BITS, GROUP, ZP, R, true, false>(a, sh);
 }
 
-// burst: up to 8 waves per workgroup, register budget for 6 waves per SIMD
+// burst: up to 8 waves per workgroup; register budget of 4 waves per SIMD (128 VGPRs), which
+// two resident workgroups per CU already reach
 template <int BITS, int GROUP, bool ZP, int R>
-__global__ void __launch_bounds__(512, 6)
+__global__ void __launch_bounds__(512, 4)
 decode_burst_kernel(const GemmArgs a, const DecodeShape sh) {
   decode_body<BITS, GROUP, ZP, R, false, false>(a, sh);
 }
