@@ -75,11 +75,17 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   while (W > 1 && W > k_tiles) { W >>= 1; S <<= 1; }
   // (group 32 carries four scales and zeros per tile and row block: two row blocks at most)
   int R = row_blocks >= 1024 ? (group_size == 32 ? 2 : 4) : 1;
-  // default prefill tile
+  // default prefill tile (measured on MI355X, Llama-3-70B layers): 32 x 128 while the batch is
+  // small enough that larger tiles would leave CUs idle, 128 x 128 beyond, and 128 x 512 for
+  // the zero-point form when its workgroups fill the 256 CUs in whole rounds
   if (!p->decode) {
-    if (M <= 32) p->cfg = 4;
-    else if (M <= 64) p->cfg = 2;
-    else p->cfg = 3;
+    if (M <= 256) {
+      p->cfg = 4;
+    } else {
+      p->cfg = 3;
+      const int64_t wgs = (N / 512) * ((M + 127) / 128);
+      if (zp && M >= 1024 && N % 512 == 0 && wgs % 256 == 0) p->cfg = 1;
+    }
   }
   if (variant != 0) {
     if (variant >= 64) {
@@ -98,6 +104,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     }
   }
   if (!p->decode) {
+    // the prefill kernel addresses X through a 32-bit buffer offset
+    if ((uint64_t)M * (uint64_t)K * 2u >= (1ull << 32)) return MATGPTQ_ESIZE;
     p->R = p->S = p->W = p->kc = 0;
     p->stream = false;
     p->smem = 0;
@@ -122,7 +130,6 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   p->stream = stream;
   p->smem = decode_lds_bytes(R, S, W, (int)kc, M);
   if (kc < k_tiles && S * W > 8) return variant != 0 ? MATGPTQ_EVARIANT : MATGPTQ_ESIZE;
-  (void)zp;
   (void)bits;
   return MATGPTQ_OK;
 }

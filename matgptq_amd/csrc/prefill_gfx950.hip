@@ -8,11 +8,23 @@
 //    packed code is dequantised by exactly one wave, straight from registers into
 //    the 16x32 MFMA operand, as  fp16(scale * fp16((c << (8-b)) - zero)),  the value
 //    the reference's dequantize() gives the weight;
-//  * the activation tile is staged through LDS (double buffered, 64 columns per
-//    stage, rows padded by 16 bytes so that the 16-byte operand reads of 16 rows
-//    fall into distinct banks) and shared by the four waves;
+//  * the activation tile is staged through LDS (two buffers of 64 columns, rows padded by
+//    16 bytes so that the 16-byte operand reads of 16 rows fall into distinct banks) and
+//    shared by the four waves; global loads of a buffer are issued four 32-column steps
+//    before their LDS store, and every global load is branch-free (tiles beyond K or N go
+//    through a zero-length buffer descriptor), so the K loop is one straight block per step;
+//  * software pipeline inside a wave: while the matrix cores work on one 32-column step, the
+//    vector ALU dequantises the next step's weights and each activation operand register is
+//    refilled from LDS as soon as the MFMAs that read it have been issued
+//    (sched_group_barrier asks the compiler for that interleaving).  The 128 x 256 tile,
+//    whose accumulators take half of a two-waves-per-SIMD register budget, runs a lean loop
+//    without the intra-wave double buffering instead;
 //  * fp32 accumulators live in registers for the whole K loop; the epilogue packs
 //    four consecutive output columns per lane into one 8-byte store.
+//
+// Measured on this target: a loop of nothing but independent MFMAs reaches 1.37 PFLOP/s with
+// one wave per SIMD and 1.91 PFLOP/s with two (nominal 2.5), which is why tiles are sized
+// for two resident waves per SIMD.
 //
 // Workgroup ids are remapped so that the workgroups of one XCD (ids congruent
 // modulo 8) walk consecutive activation tiles of the same weight rows and share
@@ -29,7 +41,10 @@ namespace {
 
 constexpr int kBits = MATGPTQ_BITS;
 constexpr int kXs = 64;          // activation columns per LDS stage
-constexpr int kXsPitch = kXs + 8;  // halves per LDS row
+#ifndef MATGPTQ_XPAD
+#define MATGPTQ_XPAD 8
+#endif
+constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 
 // One raw pair -> two weights.  u = c - 2^(b-1) is exact; with a zero point
 // v = m*u - (zero - 128) = (c << (8-b)) - zero is rounded once (exact for integral
@@ -58,8 +73,11 @@ __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const U
   a.p[3] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 3), ZP>(raw[3], zrel, scale);
 }
 
-// two waves per SIMD whenever the accumulators leave room for it
+// Two waves per SIMD (256 registers each) whenever the accumulators leave room for the rest:
+// one wave alone cannot keep the matrix pipe busy.  A tile whose accumulators take half of
+// that budget runs the lean loop below (no intra-wave double buffering).
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 <= 128 ? 2 : 1; }
+constexpr bool prefill_lean(int rbw, int mt) { return rbw * mt * 4 == 128; }
 
 template <int BITS, int GROUP, bool ZP, int RBW, int MT>
 __global__ void __launch_bounds__(256, prefill_min_waves(RBW, MT))
@@ -87,10 +105,8 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 
   constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
   const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
-  const BufRsrc wres = make_rsrc(a.packed, (uint32_t)a.row_blocks * rb_bytes);
+  const uint32_t w_bytes = (uint32_t)a.row_blocks * rb_bytes;
   const uint32_t aux_bytes = (uint32_t)a.row_blocks * a.G * 32;  // scales / zeros: [N/16][G][16] halves
-  const BufRsrc sres = make_rsrc(a.scales, aux_bytes);
-  const BufRsrc zres = make_rsrc(ZP ? a.zeros : a.scales, aux_bytes);
 
   float4v acc[RBW][MT];
 #pragma unroll
@@ -103,133 +119,197 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   _Float16 scur[RBW][GPT], snxt[RBW][GPT];
   _Float16 zcur[RBW][GPT], znxt[RBW][GPT];
 
+  // Branch-free loads: a tile beyond K, or a row block beyond N, is read through a
+  // descriptor of zero length (every lane out of range: zeros come back, nothing is fetched).
   auto load_weights = [&](uint32_t (&w)[RBW][BITS], _Float16 (&s)[RBW][GPT], _Float16 (&z)[RBW][GPT],
                           int kb) {
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
       const int rb = rb_first + rr;
 #ifdef MATGPTQ_DEBUG_NOWLOAD
-      if (rb < a.row_blocks && kb == 0) {
+      const bool valid = rb < a.row_blocks && kb == 0;
 #else
-      if (rb < a.row_blocks) {
+      const bool valid = rb < a.row_blocks && kb < a.k_tiles;
 #endif
-        load_tile_words<BITS, 0>(wres, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
+      const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
+      const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
+      const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
+      load_tile_words<BITS, 0>(wr, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
 #pragma unroll
-        for (int gg = 0; gg < GPT; gg++) {
-          const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
-          const uint32_t so = ((uint32_t)rb * a.G + g) * 32;  // bytes
-          s[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(sres, r16 * 2, so, 0));
-          if constexpr (ZP)
-            z[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(zres, r16 * 2, so, 0)) -
-                        (_Float16)128.0f;
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < BITS; i++) w[rr][i] = 0;
-#pragma unroll
-        for (int gg = 0; gg < GPT; gg++) { s[rr][gg] = (_Float16)0.0f; z[rr][gg] = (_Float16)0.0f; }
+      for (int gg = 0; gg < GPT; gg++) {
+        const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
+        const uint32_t so = ((uint32_t)rb * a.G + g) * 32;  // bytes
+        s[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0));
+        if constexpr (ZP)
+          z[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0)) -
+                      (_Float16)128.0f;
+        else
+          z[rr][gg] = (_Float16)0.0f;
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  uint4 xreg[XCHUNKS];
-  auto load_x = [&](int h) {  // columns [h*64, +64)
+  // Activation tile: two register sets, one per LDS buffer; a set is loaded four steps
+  // before it is stored.  Rows beyond M fall outside the descriptor and read as zero.
+  const uint32_t x_bytes = (uint32_t)a.M * (uint32_t)a.K * 2u;
+  uint32_t x_voff[XCHUNKS], x_lds[XCHUNKS];
 #pragma unroll
-    for (int c = 0; c < XCHUNKS; c++) {
-      const int chunk = tid + c * 256;
-      const int row = chunk >> 3, col8 = chunk & 7;
-      const int m = m0 + row;
-      xreg[c] = make_uint4(0u, 0u, 0u, 0u);
+  for (int c = 0; c < XCHUNKS; c++) {
+    const int chunk = tid + c * 256;
+    const int row = chunk >> 3, col8 = chunk & 7;
+    const uint32_t m = (uint32_t)(m0 + row);
+    x_voff[c] = m < (uint32_t)a.M ? (m * (uint32_t)a.K + col8 * 8) * 2u : x_bytes;
+    x_lds[c] = (uint32_t)(row * kXsPitch + col8 * 8);
+  }
+  u32x4 xa[XCHUNKS], xb2[XCHUNKS];
+  auto load_x = [&](u32x4 (&xr)[XCHUNKS], int h) {  // columns [h*64, +64)
 #ifdef MATGPTQ_DEBUG_NOXLOAD
-      if (m < -1)
+    const bool valid = h < 0;
 #else
-      if (m < a.M)
+    const bool valid = h < 2 * a.k_tiles;
 #endif
-        xreg[c] = *reinterpret_cast<const uint4*>(a.x + (size_t)m * a.K + (size_t)h * kXs + col8 * 8);
-    }
-  };
-  auto store_x = [&](int buf) {
+    const BufRsrc xres = make_rsrc(a.x, valid ? x_bytes : 0u);
 #pragma unroll
-    for (int c = 0; c < XCHUNKS; c++) {
-      const int chunk = tid + c * 256;
-      const int row = chunk >> 3, col8 = chunk & 7;
-      *reinterpret_cast<uint4*>(&xs[buf][row * kXsPitch + col8 * 8]) = xreg[c];
-    }
+    for (int c = 0; c < XCHUNKS; c++)
+      xr[c] = __builtin_amdgcn_raw_buffer_load_b128(xres, x_voff[c], (uint32_t)h * (kXs * 2), 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto store_x = [&](const u32x4 (&xr)[XCHUNKS], int buf) {
+#pragma unroll
+    for (int c = 0; c < XCHUNKS; c++) *reinterpret_cast<u32x4*>(&xs[buf][x_lds[c]]) = xr[c];
   };
 
-  // half step: octets J0, J0+1 of the current tile against LDS buffer `buf`.  All operand
-  // reads of a 32-column step are issued before its first MFMA, so that LDS latency is
-  // paid once per step and not once per activation tile.
-  auto half_step = [&](int buf, auto j0tag) {
-    constexpr int J0 = decltype(j0tag)::value;
-    auto k32 = [&](auto jtag) {
-      constexpr int J = decltype(jtag)::value;
-      constexpr int jj = J - J0;
-      Frag aw[RBW];
+  auto dequant_step = [&](Frag (&aw)[RBW], const uint32_t (&w)[RBW][BITS], const _Float16 (&s)[RBW][GPT],
+                          const _Float16 (&z)[RBW][GPT], auto jtag) {
+    constexpr int J = decltype(jtag)::value;
+#pragma unroll
+    for (int rr = 0; rr < RBW; rr++) {
+      const int gg = GROUP == 32 ? J : 0;
+      _Float16 s1 = s[rr][gg];
+      if constexpr (!ZP) s1 = (_Float16)((float)s1 * (float)(1 << (8 - BITS)));
+      const half2v sc = {s1, s1};
+      half2v zr = {(_Float16)0.f, (_Float16)0.f};
+      if constexpr (ZP) zr = half2v{z[rr][gg], z[rr][gg]};
+#ifdef MATGPTQ_DEBUG_NODEQUANT
+      aw[rr].u[0] = w[rr][0]; aw[rr].u[1] = w[rr][1 % BITS]; aw[rr].u[2] = w[rr][0] ^ J; aw[rr].u[3] = w[rr][1 % BITS];
+      (void)sc; (void)zr;
+#else
+      dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
+#endif
+    }
+  };
+  auto read_frag = [&](Frag& b, int i, int buf, int jj) {
+    b.v = *reinterpret_cast<const uint4*>(&xs[buf][(i * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
+  };
+  // One 32-column step of the software pipeline: the matrix cores multiply `aw` by the
+  // activation operands `b`; as soon as the MFMAs that use b[i] have been issued, b[i] is
+  // refilled with the operand of the next step (LDS buffer `nbuf`, columns [njj*32, +32)),
+  // and the vector ALU dequantises the next step's weights (`next()`) in between.  The
+  // scheduling groups ask for a few vector instructions and one LDS read after every RBW MFMAs.
+  auto step = [&](const Frag (&aw)[RBW], Frag (&b)[MT], int nbuf, int njj, auto&& next) {
+    next();
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+#pragma unroll
+      for (int rr = 0; rr < RBW; rr++)
+        acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b[i].h, acc[rr][i], 0, 0, 0);
+      read_frag(b[i], i, nbuf, njj);
+    }
+    constexpr int kValuPerMfma = (RBW * 24 + RBW * MT - 1) / (RBW * MT);
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
 #pragma unroll
       for (int rr = 0; rr < RBW; rr++) {
-        const int gg = GROUP == 32 ? J : 0;
-        _Float16 s1 = scur[rr][gg];
-        if constexpr (!ZP) s1 = (_Float16)((float)s1 * (float)(1 << (8 - BITS)));
-        const half2v sc = {s1, s1};
-        half2v zr = {(_Float16)0.f, (_Float16)0.f};
-        if constexpr (ZP) zr = half2v{zcur[rr][gg], zcur[rr][gg]};
-#ifdef MATGPTQ_DEBUG_NODEQUANT
-        aw[rr].u[0] = wcur[rr][0]; aw[rr].u[1] = wcur[rr][1 % BITS]; aw[rr].u[2] = wcur[rr][0] ^ J; aw[rr].u[3] = wcur[rr][1 % BITS];
-        (void)sc; (void)zr;
-#else
-        dequant_octet<BITS, J, ZP>(wcur[rr], kc_unpack, zr, sc, aw[rr]);
-#endif
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);  // VALU
       }
-      // activation operands in groups of four tiles: their reads are in flight together
-      constexpr int MG = MT < 4 ? MT : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if constexpr (prefill_lean(RBW, MT)) {
+    // Lean loop: one operand set, weights reloaded in place as soon as their last octet is
+    // dequantised; the other wave of the SIMD covers the latencies.
+    Frag aw[RBW];
+    auto lean_step = [&](int buf, int jj, auto jtag, auto&& after_dequant) {
+      dequant_step(aw, wcur, scur, zcur, jtag);
+      after_dequant();
+      constexpr int MG = 2;
 #pragma unroll
       for (int m0g = 0; m0g < MT; m0g += MG) {
         Frag b[MG];
 #pragma unroll
-        for (int i = 0; i < MG; i++)
-          b[i].v = *reinterpret_cast<const uint4*>(&xs[buf][((m0g + i) * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
+        for (int i = 0; i < MG; i++) read_frag(b[i], m0g + i, buf, jj);
 #pragma unroll
         for (int i = 0; i < MG; i++) {
 #pragma unroll
           for (int rr = 0; rr < RBW; rr++)
-            acc[rr][m0g + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b[i].h, acc[rr][m0g + i], 0, 0, 0);
+            acc[rr][m0g + i] =
+                __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b[i].h, acc[rr][m0g + i], 0, 0, 0);
         }
       }
     };
-    k32(std::integral_constant<int, J0>{});
-    k32(std::integral_constant<int, J0 + 1>{});
-  };
+    auto nothing = [] {};
+    load_x(xa, 0);
+    load_weights(wcur, scur, zcur, 0);
+    store_x(xa, 0);
+    __syncthreads();
+    for (int kb = 0; kb < a.k_tiles; kb++) {
+      load_x(xa, 2 * kb + 1);
+      lean_step(0, 0, std::integral_constant<int, 0>{}, nothing);
+      lean_step(0, 1, std::integral_constant<int, 1>{}, nothing);
+      store_x(xa, 1);
+      __syncthreads();
+      load_x(xa, 2 * kb + 2);
+      lean_step(1, 0, std::integral_constant<int, 2>{}, nothing);
+      lean_step(1, 1, std::integral_constant<int, 3>{}, [&] { load_weights(wcur, scur, zcur, kb + 1); });
+      store_x(xa, 0);
+      __syncthreads();
+    }
+  } else {
+  Frag awA[RBW], awB[RBW];
+  Frag bf[MT];
+  using J0 = std::integral_constant<int, 0>;
+  using J1 = std::integral_constant<int, 1>;
+  using J2 = std::integral_constant<int, 2>;
+  using J3 = std::integral_constant<int, 3>;
 
-  // prologue
-  load_x(0);
+  // prologue: half 0 into buffer 0, halves 1 and 2 into the register sets
+  load_x(xa, 0);
   load_weights(wcur, scur, zcur, 0);
-  store_x(0);
+  store_x(xa, 0);
+  load_x(xa, 1);
+  load_x(xb2, 2);
+  dequant_step(awA, wcur, scur, zcur, J0{});
   __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MT; i++) read_frag(bf[i], i, 0, 0);
 
-  const int H = a.k_tiles * 2;
   for (int kb = 0; kb < a.k_tiles; kb++) {
-    // first half of the tile
-    load_x(2 * kb + 1);
-    if (kb + 1 < a.k_tiles) load_weights(wnxt, snxt, znxt, kb + 1);
-    half_step(0, std::integral_constant<int, 0>{});
-    store_x(1);
+    load_weights(wnxt, snxt, znxt, kb + 1);
+    step(awA, bf, 0, 1, [&] { dequant_step(awB, wcur, scur, zcur, J1{}); });
+    store_x(xa, 1);  // buffer 1 was last read during step 2 of the previous tile
+    load_x(xa, 2 * kb + 3);
     __syncthreads();
-    // second half
-    if (2 * kb + 2 < H) load_x(2 * kb + 2);
-    half_step(1, std::integral_constant<int, 2>{});
-    if (2 * kb + 2 < H) store_x(0);
+    step(awB, bf, 1, 0, [&] { dequant_step(awA, wcur, scur, zcur, J2{}); });
+    step(awA, bf, 1, 1, [&] { dequant_step(awB, wcur, scur, zcur, J3{}); });
+    store_x(xb2, 0);  // buffer 0 was last read during step 0 of this tile
+    load_x(xb2, 2 * kb + 4);
     __syncthreads();
-    if (kb + 1 < a.k_tiles) {
+    // the last step of the tile prepares octet 0 of the next tile
+    step(awB, bf, 0, 0, [&] { dequant_step(awA, wnxt, snxt, znxt, J0{}); });
 #pragma unroll
-      for (int rr = 0; rr < RBW; rr++) {
+    for (int rr = 0; rr < RBW; rr++) {
 #pragma unroll
-        for (int i = 0; i < BITS; i++) wcur[rr][i] = wnxt[rr][i];
+      for (int i = 0; i < BITS; i++) wcur[rr][i] = wnxt[rr][i];
 #pragma unroll
-        for (int gg = 0; gg < GPT; gg++) { scur[rr][gg] = snxt[rr][gg]; zcur[rr][gg] = znxt[rr][gg]; }
-      }
+      for (int gg = 0; gg < GPT; gg++) { scur[rr][gg] = snxt[rr][gg]; zcur[rr][gg] = znxt[rr][gg]; }
     }
   }
+
+  }  // pipelined loop
 
   // epilogue: lane holds rows (weight rows) 4q..4q+3 of column (batch row) r16
 #pragma unroll
