@@ -40,7 +40,10 @@ COUNTER_COPY_BYTES = 256 * 1024 * 1024
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --counter-pass`, each counter scaled by what it reads for the 256 MiB elementwise copy
 # of the same run.  Keyed by the kernel plan the figure was taken on: a different plan reports null.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # FETCH_SIZE 30552.77 KiB x (262144 / 131084) + WRITE_SIZE 56 KiB x (262144 / 262144)
+    "decode-burst b4 g128 zp1 R4 S1 W8 kc32 lds40976": 62624000,
+}
 
 
 def algorithmic_bytes(n, k, m, bits, zero_points=True):
@@ -55,9 +58,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
-    ap.add_argument("--counter-pass", action="store_true",
-                    help="for rocprofv3 --pmc runs: launch only the dominant kernel over the ring of weight "
-                         "copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's yardstick)")
+    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill"),
+                    help="for rocprofv3 --pmc runs.  decode: launch only the dominant kernel over the ring of "
+                         "weight copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's "
+                         "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -116,6 +120,18 @@ def main() -> int:
         return best
 
     bits = 4
+    if args.counter_pass == "prefill":
+        n, k = LLAMA3_70B["o"]
+        packed = make_ring(n, k, bits, 1)[0]
+        sc, zr = make_aux(n, k)
+        x = torch.randn(2048, k, device=dev, generator=g).to(torch.float16)
+        y = torch.empty(2048, n, dtype=torch.float16, device=dev)
+        with torch.cuda.stream(stream):
+            for _ in range(6):
+                launch(bits, n, k, x, packed, sc, zr, y)
+            stream.synchronize()
+        print(json.dumps({"counter_pass": _lib.describe_plan(bits, GROUP, n, k, 2048, True), "launches": 6}))
+        return 0
     if args.counter_pass:
         n, k = LLAMA3_8B["gate_up"]
         copies = int(RING_BYTES // (n * k * bits // 8)) + 1
