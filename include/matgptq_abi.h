@@ -31,7 +31,7 @@ extern "C" {
 #define MATGPTQ_EGROUP (-2)    /* group_size not in {-1,32,128} or does not divide K */
 #define MATGPTQ_ESHAPE (-3)    /* N % 16 != 0, K % 128 != 0, or a size <= 0 */
 #define MATGPTQ_ENULL (-4)     /* a required pointer is NULL */
-#define MATGPTQ_EDTYPE (-5)    /* bf16 requested (flag bit 1): not built yet */
+#define MATGPTQ_EDTYPE (-5)    /* operation not available for the requested data type */
 #define MATGPTQ_ELAUNCH (-6)   /* the HIP runtime reported an error at launch */
 #define MATGPTQ_EVARIANT (-7)  /* a forced kernel variant does not apply to this problem */
 #define MATGPTQ_ESIZE (-8)     /* a size exceeds what the entry point supports */

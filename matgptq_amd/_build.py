@@ -48,11 +48,14 @@ def _run(cmd):
 def _abi_jobs():
     hipcc = _hipcc()
     jobs = []
-    for b in BITS:
-        for stem in ("decode_gfx950", "prefill_gfx950"):
-            obj = os.path.join(OBJDIR, f"{stem}_b{b}.o")
-            jobs.append((obj, [hipcc, *HIP_FLAGS, f"-DMATGPTQ_BITS={b}", "-c",
-                               os.path.join(CSRC, stem + ".hip"), "-o", obj]))
+    # the GEMM kernels are built once per bitwidth and storage type (fp16, bf16); the
+    # longest compilations go first so that the pool finishes evenly
+    for stem in ("prefill_gfx950", "decode_gfx950"):
+        for bf16 in (0, 1):
+            for b in BITS:
+                obj = os.path.join(OBJDIR, f"{stem}_b{b}{'_bf16' if bf16 else ''}.o")
+                jobs.append((obj, [hipcc, *HIP_FLAGS, f"-DMATGPTQ_BITS={b}", f"-DMATGPTQ_BF16={bf16}", "-c",
+                                   os.path.join(CSRC, stem + ".hip"), "-o", obj]))
     for stem in ("aux_gfx950", "abi"):
         obj = os.path.join(OBJDIR, stem + ".o")
         jobs.append((obj, [hipcc, *HIP_FLAGS, "-c", os.path.join(CSRC, stem + ".hip"), "-o", obj]))

@@ -17,7 +17,10 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
 #define MATGPTQ_DECL(B)                                                                        \
   hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int S, int W, int kc,  \
                                 bool stream_flavour, size_t smem, hipStream_t);                \
-  hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);
+  hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);          \
+  hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
+                                       int kc, bool stream_flavour, size_t smem, hipStream_t); \
+  hipError_t launch_prefill_b##B##_bf16(const GemmArgs&, int group_size, int cfg, hipStream_t);
 MATGPTQ_DECL(2)
 MATGPTQ_DECL(3)
 MATGPTQ_DECL(4)
@@ -134,24 +137,36 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   return MATGPTQ_OK;
 }
 
-hipError_t launch_decode(int bits, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+// `bf16`: activations, scales, zeros and output are stored as bfloat16 (same kernels built a
+// second time with the conversions at their edges)
+hipError_t launch_decode(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+#define MATGPTQ_CASE(B)                                                                      \
+  case B:                                                                                    \
+    return bf16 ? launch_decode_b##B##_bf16(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s)  \
+                : launch_decode_b##B(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
   switch (bits) {
-    case 2: return launch_decode_b2(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
-    case 3: return launch_decode_b3(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
-    case 4: return launch_decode_b4(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
-    case 6: return launch_decode_b6(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
-    default: return launch_decode_b8(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
+    MATGPTQ_CASE(2)
+    MATGPTQ_CASE(3)
+    MATGPTQ_CASE(4)
+    MATGPTQ_CASE(6)
+    default:
+      return bf16 ? launch_decode_b8_bf16(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s)
+                  : launch_decode_b8(a, g, p.R, p.S, p.W, p.kc, p.stream, p.smem, s);
   }
+#undef MATGPTQ_CASE
 }
 
-hipError_t launch_prefill(int bits, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+hipError_t launch_prefill(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+#define MATGPTQ_CASE(B) \
+  case B: return bf16 ? launch_prefill_b##B##_bf16(a, g, p.cfg, s) : launch_prefill_b##B(a, g, p.cfg, s);
   switch (bits) {
-    case 2: return launch_prefill_b2(a, g, p.cfg, s);
-    case 3: return launch_prefill_b3(a, g, p.cfg, s);
-    case 4: return launch_prefill_b4(a, g, p.cfg, s);
-    case 6: return launch_prefill_b6(a, g, p.cfg, s);
-    default: return launch_prefill_b8(a, g, p.cfg, s);
+    MATGPTQ_CASE(2)
+    MATGPTQ_CASE(3)
+    MATGPTQ_CASE(4)
+    MATGPTQ_CASE(6)
+    default: return bf16 ? launch_prefill_b8_bf16(a, g, p.cfg, s) : launch_prefill_b8(a, g, p.cfg, s);
   }
+#undef MATGPTQ_CASE
 }
 
 }  // namespace
@@ -170,7 +185,7 @@ const char* matgptq_strerror(int code) {
     case MATGPTQ_EGROUP: return "group_size must be one of {-1, 32, 128} and divide n_in_features";
     case MATGPTQ_ESHAPE: return "n_out_features must be a multiple of 16 and n_in_features a multiple of 128";
     case MATGPTQ_ENULL: return "null pointer argument";
-    case MATGPTQ_EDTYPE: return "bfloat16 is not supported by this build";
+    case MATGPTQ_EDTYPE: return "unsupported data type for this operation (float16 only)";
     case MATGPTQ_ELAUNCH: return "HIP launch failed";
     case MATGPTQ_EVARIANT: return "forced kernel variant does not apply to this problem";
     case MATGPTQ_ESIZE: return "size exceeds the supported maximum";
@@ -186,7 +201,6 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
   // the kernels address the packed tensor with 32-bit byte offsets
   if ((uint64_t)N * (uint64_t)K / 8 * (uint64_t)bitwidth >= (1ull << 32)) return MATGPTQ_ESIZE;
   if (!packed_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
-  if (flags & MATGPTQ_FLAG_BF16) return MATGPTQ_EDTYPE;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &p)) return e;
   GemmArgs a;
@@ -202,8 +216,9 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
   a.k_tiles = (int)(K / 128);
   a.row_blocks = (int)(N / 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const hipError_t err = p.decode ? launch_decode(bitwidth, a, group_size, p, s)
-                                  : launch_prefill(bitwidth, a, group_size, p, s);
+  const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
+  const hipError_t err = p.decode ? launch_decode(bitwidth, bf16, a, group_size, p, s)
+                                  : launch_prefill(bitwidth, bf16, a, group_size, p, s);
   if (err != hipSuccess) return MATGPTQ_ELAUNCH;
   if (!(flags & MATGPTQ_FLAG_ASYNC)) {
     if (hipStreamSynchronize(s) != hipSuccess) return MATGPTQ_ELAUNCH;

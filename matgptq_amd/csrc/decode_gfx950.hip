@@ -130,7 +130,7 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
             st.s[u][rr][gg] = make_uint2(sv.x, sv.y);
             if constexpr (ZP) {
               const uint16_t zv = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
-              st.z[u][rr][gg] = __builtin_bit_cast(_Float16, zv);
+              st.z[u][rr][gg] = storage_to_half(zv);
             }
           }
         }
@@ -193,6 +193,7 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
   auto x_commit = [&](XTrip& t) {
 #pragma unroll
     for (int i = 0; i < XU; i++) {
+      t.v[i] = storage8_to_half8(t.v[i]);
       scale_x(t.v[i], t.odd[i]);
       *reinterpret_cast<half8*>(xs + t.dst[i]) = t.v[i];
     }
@@ -222,15 +223,13 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
   if constexpr (!GROUPED && ZP) {
 #pragma unroll
     for (int rr = 0; rr < R; rr++)
-      zrow[rr] = live ? reinterpret_cast<const _Float16*>(a.zeros)[(size_t)(rb0 + rr) * 16 + r16]
-                      : (_Float16)128.0f;
+      zrow[rr] = live ? storage_to_half(a.zeros[(size_t)(rb0 + rr) * 16 + r16]) : (_Float16)128.0f;
   }
 
   auto fold = [&](const uint2 s4, int rr, const float4v v) {
-    H4 s;
-    s.v = s4;
+    const uint16_t sb[4] = {(uint16_t)s4.x, (uint16_t)(s4.x >> 16), (uint16_t)s4.y, (uint16_t)(s4.y >> 16)};
 #pragma unroll
-    for (int i = 0; i < 4; i++) acc[rr][i] += (float)s.h[i] * v[i];
+    for (int i = 0; i < 4; i++) acc[rr][i] += storage_to_float(sb[i]) * v[i];
   };
 
   const float4v zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -428,7 +427,7 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
       const float* src = red + ((sl * W) * R + rr) * 256 + (((row >> 2) * 16 + n) << 2) + (row & 3);
       float sum = 0.f;
       for (int w = 0; w < W; w++) sum += src[w * R * 256];
-      reinterpret_cast<_Float16*>(a.y)[(size_t)n * a.N + grow] = (_Float16)(sum * kMul);
+      a.y[(size_t)n * a.N + grow] = float_to_storage(sum * kMul);
     }
   }
 }
@@ -489,7 +488,12 @@ hipError_t launch_r(const GemmArgs& a, int R, int S, int W, int kc, bool sf, siz
 // bytes (see decode_lds_bytes in abi.hip).
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
-hipError_t MATGPTQ_CAT(launch_decode_b, MATGPTQ_BITS)(const GemmArgs& a, int group_size, int R,
+#if MATGPTQ_BF16
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(MATGPTQ_CAT(launch_decode_b, MATGPTQ_BITS), _bf16)
+#else
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_decode_b, MATGPTQ_BITS)
+#endif
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int R,
                                                       int S, int W, int kc, bool stream_flavour,
                                                       size_t smem, hipStream_t stream) {
   const bool zp = a.zeros != nullptr;

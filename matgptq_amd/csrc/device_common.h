@@ -41,6 +41,46 @@ __device__ __forceinline__ half2v h2_from_bits(uint32_t u) {
   return t.h;
 }
 
+// ---- bfloat16 storage (activations, scales, zeros, output when the BF16 flag is set) ----
+// The kernels compute in fp16 operands / fp32 accumulators either way; bf16 values are
+// converted where they enter and leave.  bf16 -> fp16 is exact inside fp16's normal range
+// (8 significant bits into 11); magnitudes above 65504 saturate to +-65504.
+#ifndef MATGPTQ_BF16
+#define MATGPTQ_BF16 0
+#endif
+constexpr bool kBf16 = MATGPTQ_BF16 != 0;
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+// 16-bit storage element (fp16 or bf16, by MATGPTQ_BF16) -> float, and float -> storage
+__device__ __forceinline__ float storage_to_float(uint16_t b) {
+  if constexpr (kBf16) return bf16_bits_to_float(b);
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+__device__ __forceinline__ uint16_t float_to_storage(float f) {
+  if constexpr (kBf16) return (uint16_t)float_to_bf16_bits(f);
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+__device__ __forceinline__ _Float16 storage_to_half(uint16_t b) {
+  if constexpr (kBf16) return (_Float16)bf16_bits_to_float(b);
+  return __builtin_bit_cast(_Float16, b);
+}
+
+// two bf16 in one word -> two fp16 (saturating)
+__device__ __forceinline__ half2v bf16x2_to_half2(uint32_t w) {
+  float lo = __uint_as_float(w << 16), hi = __uint_as_float(w & 0xffff0000u);
+  lo = __builtin_fminf(__builtin_fmaxf(lo, -65504.0f), 65504.0f);
+  hi = __builtin_fminf(__builtin_fmaxf(hi, -65504.0f), 65504.0f);
+  return half2v{(_Float16)lo, (_Float16)hi};
+}
+
 // Raw pair (1024 + c * 2^p, twice) -> (c - centre, twice), exactly.
 // (1024 + c 2^p) * 2^-p = 1024 * 2^-p + c is exact in fp16 for every p used
 // (p <= 8 and c < 2^(10-p)); so is the subtraction of the integer constant.
@@ -53,6 +93,18 @@ __device__ __forceinline__ half2v centre_raw(uint32_t raw, int centre) {
     const float inv = 1.0f / (float)(1 << P);
     return __builtin_elementwise_fma(v, h2_splat(inv), h2_splat(-(1024.0f * inv + (float)centre)));
   }
+}
+
+// eight stored activations (one 16-byte chunk) -> eight fp16
+__device__ __forceinline__ half8 storage8_to_half8(half8 raw) {
+  if constexpr (kBf16) {
+    Frag in, out;
+    in.h = raw;
+#pragma unroll
+    for (int i = 0; i < 4; i++) out.p[i] = bf16x2_to_half2(in.u[i]);
+    return out.h;
+  }
+  return raw;
 }
 
 // (x & mask) | orv.  The compiler folds this into one v_and_or_b32 when neither constant

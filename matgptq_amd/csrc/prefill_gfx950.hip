@@ -50,11 +50,14 @@ constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 // v = m*u - (zero - 128) = (c << (8-b)) - zero is rounded once (exact for integral
 // zeros) and multiplied by the scale; without, `scale` already carries the factor
 // m = 2^(8-b) (a power of two, so the single rounding of the product is unchanged).
+// bf16 storage: a bf16 scale can lie far below fp16's normal range, so the caller passes
+// scale * 2^8 (and zrel * 2^-8) and v is formed as v * 2^-8, exact as well; the
+// symmetric form takes the same route with zrel = 0.
 template <int BITS, int P, bool ZP>
 __device__ __forceinline__ half2v dequant_pair(uint32_t raw, half2v zrel, half2v scale) {
   const half2v u = centre_raw<P>(raw, Codec<BITS>::kCentre);
-  if constexpr (ZP) {
-    constexpr float m = (float)(1 << (8 - BITS));
+  if constexpr (ZP || kBf16) {
+    constexpr float m = (float)(1 << (8 - BITS)) * (kBf16 ? 1.0f / 256.0f : 1.0f);
     const half2v v = __builtin_elementwise_fma(u, h2_splat(m), -zrel);
     return v * scale;
   } else {
@@ -139,12 +142,23 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
       for (int gg = 0; gg < GPT; gg++) {
         const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
         const uint32_t so = ((uint32_t)rb * a.G + g) * 32;  // bytes
-        s[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0));
-        if constexpr (ZP)
-          z[rr][gg] = __builtin_bit_cast(_Float16, (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0)) -
-                      (_Float16)128.0f;
-        else
+        // fp16: the scale as stored (times 2^(8-b) in the symmetric form, applied below) and
+        // zero - 128; bf16: scale * 2^8 and (zero - 128) * 2^-8, converted through fp32
+        const uint16_t sbits = __builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0);
+        if constexpr (kBf16) {
+          s[rr][gg] = (_Float16)(bf16_bits_to_float(sbits) * 256.0f);
+        } else {
+          s[rr][gg] = __builtin_bit_cast(_Float16, sbits);
+        }
+        if constexpr (ZP) {
+          const uint16_t zbits = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
+          if constexpr (kBf16)
+            z[rr][gg] = (_Float16)((bf16_bits_to_float(zbits) - 128.0f) * (1.0f / 256.0f));
+          else
+            z[rr][gg] = __builtin_bit_cast(_Float16, zbits) - (_Float16)128.0f;
+        } else {
           z[rr][gg] = (_Float16)0.0f;
+        }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -177,7 +191,8 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   };
   auto store_x = [&](const u32x4 (&xr)[XCHUNKS], int buf) {
 #pragma unroll
-    for (int c = 0; c < XCHUNKS; c++) *reinterpret_cast<u32x4*>(&xs[buf][x_lds[c]]) = xr[c];
+    for (int c = 0; c < XCHUNKS; c++)
+      *reinterpret_cast<half8*>(&xs[buf][x_lds[c]]) = storage8_to_half8(__builtin_bit_cast(half8, xr[c]));
   };
 
   auto dequant_step = [&](Frag (&aw)[RBW], const uint32_t (&w)[RBW][BITS], const _Float16 (&s)[RBW][GPT],
@@ -187,7 +202,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     for (int rr = 0; rr < RBW; rr++) {
       const int gg = GROUP == 32 ? J : 0;
       _Float16 s1 = s[rr][gg];
-      if constexpr (!ZP) s1 = (_Float16)((float)s1 * (float)(1 << (8 - BITS)));
+      if constexpr (!ZP && !kBf16) s1 = (_Float16)((float)s1 * (float)(1 << (8 - BITS)));
       const half2v sc = {s1, s1};
       half2v zr = {(_Float16)0.f, (_Float16)0.f};
       if constexpr (ZP) zr = half2v{z[rr][gg], z[rr][gg]};
@@ -320,10 +335,11 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     for (int mt = 0; mt < MT; mt++) {
       const int m = m0 + mt * 16 + r16;
       if (m < a.M) {
-        H4 o;
+        uint16_t o[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) o.h[i] = (_Float16)acc[rr][mt][i];
-        *reinterpret_cast<uint2*>(a.y + (size_t)m * a.N + (size_t)rb * 16 + 4 * q) = o.v;
+        for (int i = 0; i < 4; i++) o[i] = float_to_storage(acc[rr][mt][i]);
+        *reinterpret_cast<uint2*>(a.y + (size_t)m * a.N + (size_t)rb * 16 + 4 * q) =
+            make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
       }
     }
   }
@@ -358,7 +374,12 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 // cfg selects the workgroup tile (see launch_shape).
-hipError_t MATGPTQ_CAT(launch_prefill_b, MATGPTQ_BITS)(const GemmArgs& a, int group_size, int cfg,
+#if MATGPTQ_BF16
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(MATGPTQ_CAT(launch_prefill_b, MATGPTQ_BITS), _bf16)
+#else
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_prefill_b, MATGPTQ_BITS)
+#endif
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int cfg,
                                                        hipStream_t stream) {
   const bool zp = a.zeros != nullptr;
   if (group_size == 128)

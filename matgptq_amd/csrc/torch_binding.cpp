@@ -144,9 +144,11 @@ Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& sca
   TORCH_CHECK(weights.size(0) == bitwidth * n_out_features * n_in_features / 32,
               "matgptq_weights has the wrong size");
   const bool bf16 = (feature_flag & MATGPTQ_FLAG_BF16) != 0;
-  TORCH_CHECK(!bf16, "matmul_matgptq: bfloat16 is not supported by this build (float16 only)");
-  TORCH_CHECK(input.dtype() == torch::kFloat16, "matmul_matgptq: input must be float16");
-  TORCH_CHECK(scales.dtype() == torch::kFloat16, "matmul_matgptq: matgptq_scales must be float16");
+  // the reference trusts the flag (bindings.cpp:171-174); a mismatch is reported here
+  const auto want = bf16 ? torch::kBFloat16 : torch::kFloat16;
+  const char* want_name = bf16 ? "bfloat16 (feature_flag bit 1 is set)" : "float16 (feature_flag bit 1 is clear)";
+  TORCH_CHECK(input.dtype() == want, "matmul_matgptq: input must be ", want_name);
+  TORCH_CHECK(scales.dtype() == want, "matmul_matgptq: matgptq_scales must be ", want_name);
   TORCH_CHECK(input.dim() >= 2 && input.size(-1) == n_in_features,
               "matmul_matgptq: input must be (..., batch, n_in_features)");
   TORCH_CHECK(input.is_contiguous(), "matmul_matgptq: input must be contiguous");
@@ -157,7 +159,7 @@ Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& sca
   if (zeros.has_value()) {
     const Tensor& z = *zeros;
     TORCH_CHECK(z.is_cuda() && z.device() == input.device(), "matgptq_zeros must be on the GPU of the input");
-    TORCH_CHECK(z.dtype() == torch::kFloat16, "matgptq_zeros must be float16");
+    TORCH_CHECK(z.dtype() == want, "matgptq_zeros must be ", want_name);
     TORCH_CHECK(z.is_contiguous() && z.numel() == n_out_features * groups,
                 "matgptq_zeros has the wrong size");
     zeros_ptr = z.data_ptr();

@@ -25,6 +25,12 @@ How each function is pinned (see tests/test_oracle.py):
   * linear           float64 matmul of the fp16-rounded weight (library routine);
                      in the reference test's regime (0/1 scales, integer x) the
                      result is exact and is compared for equality.
+  * bfloat16 forms   (round_to_bf16, dequantize_bf16, fake_matryoshka_linear_bf16)
+                     rounding: exhaustive comparison with torch's float32 -> bfloat16
+                     conversion on all 2^16 upper halves x three lower-half patterns
+                     (tie, below, above); dequantize / forward: the committed golden
+                     vectors the reference's dequantize and FakeMatryoshkaLinear give
+                     on bfloat16 tensors.
 """
 from __future__ import annotations
 
@@ -115,6 +121,51 @@ def fake_matryoshka_linear(x: np.ndarray, q: np.ndarray, scale: np.ndarray, zero
                            master_bits: int = MASTER_BITS) -> np.ndarray:
     """FakeMatryoshkaLinear.forward without perm/bias (src/quant_utils_matgpqt.py:202-224)."""
     return linear(x, dequantize(q, scale, zero, slice_bits, group_size, master_bits))
+
+
+# --------------------------------------------------------------------------
+# bfloat16 storage (feature flag bit 1 of the reference, common.cuh:78-86): the same
+# formulas evaluated on bfloat16 tensors.  bfloat16 values are carried as float32 here.
+# --------------------------------------------------------------------------
+
+def round_to_bf16(a: np.ndarray) -> np.ndarray:
+    """float -> nearest bfloat16 (ties to even), returned as float32."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    r = np.where(nan, 0x7FC00000, r).astype(np.uint32)
+    return r.view(np.float32)
+
+
+def bf16_bits(a: np.ndarray) -> np.ndarray:
+    """bfloat16-representable float32 -> uint16 bit patterns."""
+    return (np.ascontiguousarray(a, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_from_bits(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def dequantize_bf16(q: np.ndarray, scale: np.ndarray, zero: np.ndarray, slice_bits: int,
+                    group_size: int, master_bits: int = MASTER_BITS) -> np.ndarray:
+    """`dequantize` on bfloat16 tensors (src/quant_utils_matgpqt.py:19-22): the difference
+    `q_shifted - zero` and the product with `scale` are each rounded to bfloat16.
+    `scale`, `zero`: bfloat16 values held in float32.  Returns float32 holding bfloat16."""
+    n, k = q.shape
+    s = slice_codes(q, slice_bits, master_bits).astype(np.int32) << (master_bits - slice_bits)
+    z = _expand_groups(np.asarray(zero, dtype=np.float32), n, k, group_size)
+    sc = _expand_groups(np.asarray(scale, dtype=np.float32), n, k, group_size)
+    diff = round_to_bf16(s.astype(np.float64) - z.astype(np.float64))
+    # an 8-bit by 8-bit significand product is exact in float32: one rounding to bfloat16
+    return round_to_bf16(sc.astype(np.float32) * diff)
+
+
+def fake_matryoshka_linear_bf16(x: np.ndarray, q: np.ndarray, scale: np.ndarray, zero: np.ndarray,
+                                slice_bits: int, group_size: int,
+                                master_bits: int = MASTER_BITS) -> np.ndarray:
+    """FakeMatryoshkaLinear.forward on bfloat16 tensors: wide accumulation, one rounding."""
+    w = dequantize_bf16(q, scale, zero, slice_bits, group_size, master_bits)
+    return round_to_bf16(linear_f64(x, w))
 
 
 def abs_product_bound(x: np.ndarray, w: np.ndarray) -> np.ndarray:

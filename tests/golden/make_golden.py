@@ -72,6 +72,25 @@ def main() -> None:
         w = ref.dequantize(q.view(n, k // gs2, gs2), scale2.view(n, -1, 1), zero2.view(n, -1, 1), 8, 3)
         out[f"w_b3_{tag}"] = w.reshape(n, k).numpy()
 
+    # 5. the same functions on bfloat16 tensors (feature flag bit 1); values are stored as
+    #    float32, which holds every bfloat16 exactly
+    g5 = torch.Generator().manual_seed(4321)
+    scale_bf = (torch.randn(n, k // gs, generator=g5).abs() * 0.01 + 1e-3).to(torch.bfloat16)
+    zero_bf = torch.randint(0, 256, (n, k // gs), generator=g5).to(torch.bfloat16)
+    x_bf = torch.randn(3, k, generator=g5).to(torch.bfloat16)
+    out["scale_bf16"] = scale_bf.float().numpy()
+    out["zero_bf16"] = zero_bf.float().numpy()
+    out["x_bf16"] = x_bf.float().numpy()
+    for b in BITS:
+        w = ref.dequantize(q.view(n, k // gs, gs), scale_bf.view(n, -1, 1), zero_bf.view(n, -1, 1), 8, b)
+        assert w.dtype == torch.bfloat16
+        out[f"w_bf16_b{b}"] = w.reshape(n, k).float().numpy()
+        layer = _build_layer(ref, q, scale_bf, zero_bf, b)
+        with torch.no_grad():
+            y = layer(x_bf)
+        assert y.dtype == torch.bfloat16
+        out[f"y_bf16_b{b}"] = y.float().numpy()
+
     dst = os.path.join(os.path.dirname(os.path.abspath(__file__)), "matgptq_golden.npz")
     np.savez_compressed(dst, **out)
     print("wrote", dst, {k_: v.shape for k_, v in out.items()})

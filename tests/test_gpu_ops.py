@@ -36,6 +36,22 @@ def test_module_like_the_reference_test(b):
         G.assert_close_to_oracle(y.cpu().numpy(), x, w, f"module b={b} M={m}")
 
 
+def test_module_bfloat16():
+    # bf16 scales select the bf16 flag (matgptq_linear.py:26 of the reference); output is bf16
+    n, k, g, b = 64, 1024, 128, 4
+    q, s16, _ = o.make_layer(n, k, g, seed=9, symmetric=True)
+    s = o.round_to_bf16(s16.astype(np.float32))
+    lin = MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)), torch.from_numpy(s).to(torch.bfloat16), b, g)
+    assert lin.flag == 3 and lin.matgptq_scales.dtype == torch.bfloat16
+    w = o.dequantize_bf16(q, s, np.full_like(s, 128.0), b, g)
+    for m in (1, 8, 33):
+        x = o.round_to_bf16(o.make_activations(m, k, seed=m).astype(np.float32))
+        y = lin(torch.from_numpy(x).to(torch.bfloat16).cuda())
+        assert y.shape == (m, n) and y.dtype == torch.bfloat16
+        ref = o.linear_f64(x, w)
+        assert np.max(np.abs(y.float().cpu().numpy() - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+
+
 def test_ops_accept_device_tensors_and_match_host_packing():
     n, k, b, g = 48, 512, 3, 32
     q, s, z = o.make_layer(n, k, g, seed=2)
@@ -74,10 +90,14 @@ def test_op_errors_on_device():
         mm(x, w.view(torch.int32), s, n, k, 4, 128, 1)
     with pytest.raises(RuntimeError, match="bitwidth must be one of"):
         mm(x, w, s, n, k, 5, 128, 1)
-    with pytest.raises(RuntimeError, match="bfloat16"):
-        mm(x.to(torch.bfloat16), w, s.to(torch.bfloat16), n, k, 4, 128, 3)
+    with pytest.raises(RuntimeError, match="input must be bfloat16"):
+        mm(x, w, s, n, k, 4, 128, 3)  # flag says bf16, tensors are fp16
+    with pytest.raises(RuntimeError, match="input must be float16"):
+        mm(x.to(torch.bfloat16), w, s.to(torch.bfloat16), n, k, 4, 128, 1)
     with pytest.raises(RuntimeError, match="input must be float16"):
         mm(x.float(), w, s, n, k, 4, 128, 1)
+    yb = mm(x.to(torch.bfloat16), w, s.to(torch.bfloat16), n, k, 4, 128, 3)
+    assert yb.dtype == torch.bfloat16 and yb.shape == (1, n)
     assert mm(x[:0], w, s, n, k, 4, 128, 1).shape == (0, n)  # empty batch
 
 

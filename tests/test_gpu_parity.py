@@ -206,5 +206,79 @@ def test_sync_flag_and_error_paths_on_device():
     assert np.array_equal(y_async, y_sync)
     with pytest.raises(_lib.MatGPTQError, match="variant"):
         lay.run(x, flags=1 | (200 << 8))
-    with pytest.raises(_lib.MatGPTQError, match="bfloat16"):
-        lay.run(x, flags=3)
+
+
+# ---------------------------------------------------------------- bfloat16 storage (flag bit 1)
+
+def _bf16_dev(a_f32: np.ndarray) -> torch.Tensor:
+    """float32 array of bfloat16-representable values -> bfloat16 tensor on the device."""
+    return torch.from_numpy(np.ascontiguousarray(a_f32, dtype=np.float32)).to(torch.bfloat16).to(G.DEV)
+
+
+def _gemm_bf16(b, g, n, k, x_f32, packed, s_f32, z_f32, flags=3):
+    L = G.lib()
+    xd = _bf16_dev(x_f32)
+    sd = _bf16_dev(s_f32)
+    sr = torch.empty_like(sd)
+    _lib.check(L.matgptq_reorder_scales_device(sd.data_ptr(), n, k, g, sr.data_ptr(), G.stream()))
+    zr = None
+    if z_f32 is not None:
+        zd = _bf16_dev(z_f32)
+        zr = torch.empty_like(zd)
+        _lib.check(L.matgptq_reorder_scales_device(zd.data_ptr(), n, k, g, zr.data_ptr(), G.stream()))
+    y = torch.empty(xd.shape[0], n, dtype=torch.bfloat16, device=G.DEV)
+    _lib.check(L.matgptq_gemm(b, g, n, k, xd.shape[0], packed.data_ptr(), sr.data_ptr(),
+                              zr.data_ptr() if zr is not None else None, xd.data_ptr(), y.data_ptr(),
+                              G.stream(), flags))
+    torch.cuda.synchronize()
+    return y.float().cpu().numpy()
+
+
+# One bfloat16 rounding of the output is 2^-9 relative; the oracle additionally rounds every
+# weight to bfloat16 (2^-9 each, independent), which the kernels do not (they keep fp16 weights /
+# exact products).  Bar: max error <= 1e-2 of the largest output, as for fp16.
+@pytest.mark.parametrize("b", BITS)
+def test_bf16_forward_against_reference_vectors(b, golden):
+    n, k = golden["q"].shape
+    pk = G.pack_device(golden["q"], b, True)
+    y = _gemm_bf16(b, 128, n, k, golden["x_bf16"], pk, golden["scale_bf16"], golden["zero_bf16"])
+    ref = golden[f"y_bf16_b{b}"].astype(np.float64)
+    assert np.all(np.isfinite(y))
+    assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("m", (1, 5, 16, 40, 200))
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_bf16_gemm_matches_oracle(b, g, m):
+    n, k = 96, 1024
+    q, s16, z16 = o.make_layer(n, k, g, seed=3 * b + m)
+    s = o.round_to_bf16(s16.astype(np.float32))
+    z = z16.astype(np.float32)  # integers up to 255: bfloat16 values
+    x = o.round_to_bf16(o.make_activations(m, k, seed=m + b, outlier_frac=0.01).astype(np.float32))
+    pk = G.pack_device(q, b, True)
+    for zeros in (z, None):
+        zz = z if zeros is not None else np.full_like(z, 128.0)
+        y = _gemm_bf16(b, g, n, k, x, pk, s, zeros)
+        w = o.dequantize_bf16(q, s, zz, b, g)
+        ref = o.linear_f64(x, w)
+        assert np.all(np.isfinite(y))
+        err = np.abs(y - ref)
+        assert err.max() <= G.REL_TOL * np.max(np.abs(ref)), (b, g, m, zeros is None, err.max())
+        # output values are bfloat16
+        assert np.array_equal(o.round_to_bf16(y), y)
+
+
+def test_bf16_small_scales_and_large_activations():
+    # scales far below fp16's normal range and activations at the top of it
+    n, k, b, g = 64, 512, 4, 128
+    q, _, z16 = o.make_layer(n, k, g, seed=11)
+    s = o.round_to_bf16(np.full((n, k // g), 3e-7, dtype=np.float32))
+    z = z16.astype(np.float32)
+    x = o.round_to_bf16((o.make_activations(48, k, seed=2).astype(np.float32)) * 8000.0)
+    pk = G.pack_device(q, b, True)
+    for rows in (slice(0, 3), slice(0, 48)):  # decode and prefill kernels
+        y = _gemm_bf16(b, g, n, k, x[rows], pk, s, z)
+        ref = o.linear_f64(x[rows], o.dequantize_bf16(q, s, z, b, g))
+        assert np.all(np.isfinite(y))
+        assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref))

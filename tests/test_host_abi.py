@@ -119,7 +119,6 @@ def test_error_codes():
     assert lib.matgptq_gemm(7, 128, 16, 128, 1, 1, 1, None, 1, 1, None, 1) == -1
     assert lib.matgptq_gemm(4, 48, 16, 128, 1, 1, 1, None, 1, 1, None, 1) == -2
     assert lib.matgptq_gemm(4, 128, 16, 128, 0, 1, 1, None, 1, 1, None, 1) == -8
-    assert lib.matgptq_gemm(4, 128, 16, 128, 1, 1, 1, None, 1, 1, None, 3) == -5  # bf16
     for code in range(-8, 1):
         assert lib.matgptq_strerror(code)
     with pytest.raises(_lib.MatGPTQError, match="bitwidth must be one of"):

@@ -129,3 +129,44 @@ def test_c_oracle_matches_numpy_on_random_layer():
         a = o.fake_matryoshka_linear(x, q, s, z, b, 128)
         c = c_oracle.forward(x, q, s, z, b, 128)
         assert np.array_equal(a.view(np.uint16), c.view(np.uint16))
+
+
+# ---------------------------------------------------------------- bfloat16 forms
+
+def test_bf16_rounding_matches_torch_exhaustively():
+    import torch
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    for lo in (0x0000, 0x7FFF, 0x8000, 0x8001, 0xFFFF):
+        a = (hi | lo).view(np.float32)
+        mine = o.round_to_bf16(a)
+        ref = torch.from_numpy(a.copy()).to(torch.bfloat16).float().numpy()
+        nan = np.isnan(ref)
+        assert np.array_equal(np.isnan(mine), nan)
+        assert np.array_equal(mine[~nan].view(np.uint32), ref[~nan].view(np.uint32)), hex(lo)
+    assert np.array_equal(o.bf16_from_bits(o.bf16_bits(mine[~nan])), mine[~nan])
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_bf16_dequantize_and_forward_match_golden(b, golden):
+    w = o.dequantize_bf16(golden["q"], golden["scale_bf16"], golden["zero_bf16"], b, 128)
+    assert np.array_equal(w.view(np.uint32), golden[f"w_bf16_b{b}"].view(np.uint32))
+    y = o.fake_matryoshka_linear_bf16(golden["x_bf16"], golden["q"], golden["scale_bf16"],
+                                      golden["zero_bf16"], b, 128)
+    ref = golden[f"y_bf16_b{b}"].astype(np.float64)
+    # torch accumulates the bfloat16 product in fp32: within one bfloat16 step of the value
+    assert np.max(np.abs(y - ref)) <= 2.0 ** -7 * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("b", BITS)
+def test_bf16_torch_path_matches_golden(b, golden):
+    import torch
+    from oracle import torch_path
+    q = torch.from_numpy(golden["q"])
+    s = torch.from_numpy(golden["scale_bf16"]).to(torch.bfloat16)
+    z = torch.from_numpy(golden["zero_bf16"]).to(torch.bfloat16)
+    x = torch.from_numpy(golden["x_bf16"]).to(torch.bfloat16)
+    w = torch_path.get_weight(q, s, z, 8, b)
+    assert w.dtype == torch.bfloat16
+    assert np.array_equal(w.float().numpy().view(np.uint32), golden[f"w_bf16_b{b}"].view(np.uint32))
+    y = torch_path.forward(x, q, s, z, 8, b)
+    assert np.array_equal(y.float().numpy().view(np.uint32), golden[f"y_bf16_b{b}"].view(np.uint32))
