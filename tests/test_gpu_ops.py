@@ -153,3 +153,45 @@ def test_vllm_linear_method_matches_module(with_zeros):
     lin = MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)).cuda(), torch.from_numpy(s).cuda(), b, g,
                         zeros=torch.from_numpy(z).cuda() if with_zeros else None)
     assert torch.equal(lin(torch.from_numpy(x.reshape(6, k)).cuda()) + bias, y.view(6, -1))
+
+
+@pytest.mark.parametrize("with_zeros", (False, True))
+def test_packed_checkpoint_to_module(tmp_path, with_zeros):
+    # write a packed checkpoint, read it back, build the modules the transformers demo builds
+    # (inference_demo_transformers.py:30-62), compare with the oracle on the stored tensors
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    from matgptq_amd import checkpoint as ck
+
+    model, quant, out = str(tmp_path / "m"), str(tmp_path / "q"), str(tmp_path / "out")
+    os.makedirs(model)
+    shapes = {"model.layers.0.mlp.up_proj": (64, 512), "model.layers.0.mlp.down_proj": (48, 1024)}
+    save_file({f"{k}.weight": torch.zeros(n, kk).half() for k, (n, kk) in shapes.items()},
+              os.path.join(model, ck.SINGLE_NAME))
+    with open(os.path.join(model, "config.json"), "w") as f:
+        json.dump({}, f)
+    layers = {}
+    for i, (name, (n, k)) in enumerate(shapes.items()):
+        q, s, z = o.make_layer(n, k, 128, seed=20 + i, symmetric=not with_zeros)
+        data = {"qweight": torch.from_numpy(q), "scale": torch.from_numpy(s)}
+        if with_zeros:
+            data["zero"] = torch.from_numpy(z)
+        os.makedirs(os.path.join(quant, name))
+        torch.save(data, os.path.join(quant, name, "data.pt"))
+        layers[name] = (q, s, z)
+    ck.pack_model(model, quant, out, 128, 8, 4, "float16", layer_bitwidths={"down_proj": 3})
+    qc = ck.read_quantization_config(out)
+    seen = 0
+    for name, tensors in ck.iter_quantised_layers(out):
+        bits = ck.bitwidth_of(name, qc)
+        assert bits == (3 if name.endswith("down_proj") else 4)
+        lin = ck.build_linear(tensors, bits, qc)
+        q, s, z = layers[name]
+        x = o.make_activations(5, q.shape[1], seed=seen)
+        y = lin(torch.from_numpy(x).cuda())
+        G.assert_close_to_oracle(y.cpu().numpy(), x, o.dequantize(q, s, z, bits, 128), name)
+        seen += 1
+    assert seen == 2
