@@ -235,6 +235,27 @@ def main() -> int:
         extra["small_batch"] = small
         del rings
         torch.cuda.empty_cache()
+        # ------------------------------------------- Mix'n'Match decode step (configs[3])
+        # the 128 linears of a 32-layer Llama-3-8B-shaped decoder at batch 1, every linear at a
+        # bitwidth drawn from {2,3,4,6,8} (seeded); attention, norms and the head are not part
+        # of the measured path, so this is the linear share of a token, not end-to-end tokens/s
+        import random
+        rnd = random.Random(0)
+        stack, total_bytes, hist = [], 0, {}
+        for _layer in range(32):
+            for name, (n, k) in LLAMA3_8B.items():
+                b = rnd.choice((2, 3, 4, 6, 8))
+                hist[b] = hist.get(b, 0) + 1
+                stack.append((b, n, k, xs[name], make_ring(n, k, b, 1)[0], aux[name][0], aux[name][1], ys[name]))
+                total_bytes += n * k * b // 8
+        t = timed_graph(lambda: [launch(*item) for item in stack])
+        extra["mixnmatch_decode_linears"] = {
+            "linears": len(stack), "bitwidth_histogram": {str(b): c for b, c in sorted(hist.items())},
+            "mean_bits": round(total_bytes * 8 / sum(n * k for _, n, k, *_ in stack), 2),
+            "ms_per_token": round(t * 1e3, 4), "tokens_per_s_linears_only": round(1.0 / t, 1),
+            "weight_GBps": round(total_bytes / t / 1e9, 1)}
+        del stack
+        torch.cuda.empty_cache()
         # --------------------------------------------------------------- prefill
         pre = {}
         m = 2048

@@ -282,3 +282,24 @@ def test_bf16_small_scales_and_large_activations():
         ref = o.linear_f64(x[rows], o.dequantize_bf16(q, s, z, b, g))
         assert np.all(np.isfinite(y))
         assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("gsz", GROUPS)
+@pytest.mark.parametrize("m", (1, 8, 16))
+@pytest.mark.parametrize("k", (1024, 4096, 8192))
+@pytest.mark.parametrize("b", BITS)
+def test_reference_kernel_test_grid_bf16(b, k, m, gsz):
+    # the bfloat16 half of the reference's test grid (inference_lib/test_matgptq_matmul.py:11-49):
+    # every product and partial sum is an integer below 2^24, so the fp32 accumulation is exact
+    # and the output must be the bfloat16 rounding of the closed form, bit for bit.
+    rng = np.random.default_rng(2)
+    n = 16
+    g = k if gsz == -1 else gsz
+    codes = rng.integers(0, 1 << b, (n, k), dtype=np.uint8)
+    scales = np.round(rng.random((n, k // g))).astype(np.float32)
+    x = np.round(rng.standard_normal((m, k))).astype(np.float32)
+    w = (codes.astype(np.float64) - (1 << (b - 1))) * np.repeat(scales, g, axis=1) * (1 << (8 - b))
+    expect = o.round_to_bf16(o.linear_f64(x, w))
+    pk = G.pack_device(codes, b, from_master=False)
+    y = _gemm_bf16(b, gsz, n, k, x, pk, scales, None)
+    assert np.array_equal(y.view(np.uint32), expect.view(np.uint32))
