@@ -78,6 +78,12 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   while (W > 1 && W > k_tiles) { W >>= 1; S <<= 1; }
   // (group 32 carries four scales and zeros per tile and row block: two row blocks at most)
   int R = row_blocks >= 1024 ? (group_size == 32 ? 2 : 4) : 1;
+  // from four batch rows on, the copy of X' each workgroup stages starts to count: more row
+  // blocks per workgroup (two slots of two, or two per wave) amortise it better
+  if (M >= 4 && k_tiles >= 8) {
+    if (row_blocks >= 1024) { R = 2; S = 2; W = 4; }
+    else if (row_blocks >= 320) { R = 2; }
+  }
   // default prefill tile (measured on MI355X, Llama-3-70B layers): 32 x 128 while the batch is
   // small enough that larger tiles would leave CUs idle, 128 x 128 beyond, and 128 x 512 for
   // the zero-point form when its workgroups fill the 256 CUs in whole rounds
