@@ -10,8 +10,8 @@
 //    the reference's dequantize() gives the weight;
 //  * the activation tile is staged through LDS (two buffers of 64 columns, rows padded by
 //    16 bytes so that the 16-byte operand reads of 16 rows fall into distinct banks) and
-//    shared by the four waves; global loads of a buffer are issued four 32-column steps
-//    before their LDS store, and every global load is branch-free (tiles beyond K or N go
+//    shared by the four waves; global loads of a buffer are issued eight 32-column steps
+//    (four for the largest tile) before their LDS store, and every global load is branch-free (tiles beyond K or N go
 //    through a zero-length buffer descriptor), so the K loop is one straight block per step;
 //  * software pipeline inside a wave: while the matrix cores work on one 32-column step, the
 //    vector ALU dequantises the next step's weights and each activation operand register is
@@ -176,7 +176,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     x_voff[c] = m < (uint32_t)a.M ? (m * (uint32_t)a.K + col8 * 8) * 2u : x_bytes;
     x_lds[c] = (uint32_t)(row * kXsPitch + col8 * 8);
   }
-  u32x4 xa[XCHUNKS], xb2[XCHUNKS];
+  u32x4 xa[XCHUNKS];  // the lean loop's single set
   auto load_x = [&](u32x4 (&xr)[XCHUNKS], int h) {  // columns [h*64, +64)
 #ifdef MATGPTQ_DEBUG_NOXLOAD
     const bool valid = h < 0;
@@ -291,36 +291,82 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   using J2 = std::integral_constant<int, 2>;
   using J3 = std::integral_constant<int, 3>;
 
-  // prologue: half 0 into buffer 0, halves 1 and 2 into the register sets
-  load_x(xa, 0);
-  load_weights(wcur, scur, zcur, 0);
-  store_x(xa, 0);
-  load_x(xa, 1);
-  load_x(xb2, 2);
-  dequant_step(awA, wcur, scur, zcur, J0{});
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < MT; i++) read_frag(bf[i], i, 0, 0);
+  if constexpr (RBW * MT * 4 >= 256) {
+    // the accumulators fill the accumulation registers: one tile per trip, activations two
+    // half tiles ahead, weights one tile ahead
+    u32x4 xo[2][XCHUNKS];
+    // prologue: half 0 into buffer 0, halves 1 and 2 into the register sets
+    load_x(xo[0], 0);
+    load_weights(wcur, scur, zcur, 0);
+    store_x(xo[0], 0);
+    load_x(xo[0], 1);
+    load_x(xo[1], 2);
+    dequant_step(awA, wcur, scur, zcur, J0{});
+    __syncthreads();
+  #pragma unroll
+    for (int i = 0; i < MT; i++) read_frag(bf[i], i, 0, 0);
 
-  for (int kb = 0; kb < a.k_tiles; kb++) {
-    load_weights(wnxt, snxt, znxt, kb + 1);
-    step(awA, bf, 0, 1, [&] { dequant_step(awB, wcur, scur, zcur, J1{}); });
-    store_x(xa, 1);  // buffer 1 was last read during step 2 of the previous tile
-    load_x(xa, 2 * kb + 3);
+    for (int kb = 0; kb < a.k_tiles; kb++) {
+      load_weights(wnxt, snxt, znxt, kb + 1);
+      step(awA, bf, 0, 1, [&] { dequant_step(awB, wcur, scur, zcur, J1{}); });
+      store_x(xo[0], 1);  // buffer 1 was last read during step 2 of the previous tile
+      load_x(xo[0], 2 * kb + 3);
+      __syncthreads();
+      step(awB, bf, 1, 0, [&] { dequant_step(awA, wcur, scur, zcur, J2{}); });
+      step(awA, bf, 1, 1, [&] { dequant_step(awB, wcur, scur, zcur, J3{}); });
+      store_x(xo[1], 0);  // buffer 0 was last read during step 0 of this tile
+      load_x(xo[1], 2 * kb + 4);
+      __syncthreads();
+      // the last step of the tile prepares octet 0 of the next tile
+      step(awB, bf, 0, 0, [&] { dequant_step(awA, wnxt, snxt, znxt, J0{}); });
+  #pragma unroll
+      for (int rr = 0; rr < RBW; rr++) {
+  #pragma unroll
+        for (int i = 0; i < BITS; i++) wcur[rr][i] = wnxt[rr][i];
+  #pragma unroll
+        for (int gg = 0; gg < GPT; gg++) { scur[rr][gg] = snxt[rr][gg]; zcur[rr][gg] = znxt[rr][gg]; }
+      }
+    }
+  } else {
+    // Register sets of the activation prefetch: half tile h travels in set h % NX and is
+    // loaded NX half tiles (2 NX steps) before it is stored to LDS.  Weights: two sets (even
+    // and odd tiles); a set is reloaded for the tile after next as soon as its last octet
+    // has been dequantised, five steps before that tile's first octet is needed.
+    constexpr int NX = 4;
+    u32x4 xr[NX][XCHUNKS];
+    load_x(xr[0], 0);
+    load_weights(wcur, scur, zcur, 0);
+    load_weights(wnxt, snxt, znxt, 1);
+    store_x(xr[0], 0);
+  #pragma unroll
+    for (int h = 1; h <= NX; h++) load_x(xr[h & (NX - 1)], h);
+    dequant_step(awA, wcur, scur, zcur, J0{});
     __syncthreads();
-    step(awB, bf, 1, 0, [&] { dequant_step(awA, wcur, scur, zcur, J2{}); });
-    step(awA, bf, 1, 1, [&] { dequant_step(awB, wcur, scur, zcur, J3{}); });
-    store_x(xb2, 0);  // buffer 0 was last read during step 0 of this tile
-    load_x(xb2, 2 * kb + 4);
-    __syncthreads();
-    // the last step of the tile prepares octet 0 of the next tile
-    step(awB, bf, 0, 0, [&] { dequant_step(awA, wnxt, snxt, znxt, J0{}); });
-#pragma unroll
-    for (int rr = 0; rr < RBW; rr++) {
-#pragma unroll
-      for (int i = 0; i < BITS; i++) wcur[rr][i] = wnxt[rr][i];
-#pragma unroll
-      for (int gg = 0; gg < GPT; gg++) { scur[rr][gg] = snxt[rr][gg]; zcur[rr][gg] = znxt[rr][gg]; }
+  #pragma unroll
+    for (int i = 0; i < MT; i++) read_frag(bf[i], i, 0, 0);
+
+    // one tile: weights `wc` (the next tile's are in `wn`), activation sets `sa` / `sb` for
+    // the half tiles 2 kb + 1 (LDS buffer 1) and 2 kb + 2 (buffer 0)
+    auto tile = [&](int kb, uint32_t (&wc)[RBW][BITS], _Float16 (&sc)[RBW][GPT], _Float16 (&zc)[RBW][GPT],
+                    const uint32_t (&wn)[RBW][BITS], const _Float16 (&sn)[RBW][GPT],
+                    const _Float16 (&zn)[RBW][GPT], u32x4 (&sa)[XCHUNKS], u32x4 (&sb)[XCHUNKS]) {
+      step(awA, bf, 0, 1, [&] { dequant_step(awB, wc, sc, zc, J1{}); });
+      store_x(sa, 1);  // buffer 1 was last read during step 2 of the previous tile
+      load_x(sa, 2 * kb + 1 + NX);
+      __syncthreads();
+      step(awB, bf, 1, 0, [&] { dequant_step(awA, wc, sc, zc, J2{}); });
+      step(awA, bf, 1, 1, [&] { dequant_step(awB, wc, sc, zc, J3{}); });
+      load_weights(wc, sc, zc, kb + 2);  // this set is free now
+      store_x(sb, 0);  // buffer 0 was last read during step 0 of this tile
+      load_x(sb, 2 * kb + 2 + NX);
+      __syncthreads();
+      // the last step of the tile prepares octet 0 of the next tile
+      step(awB, bf, 0, 0, [&] { dequant_step(awA, wn, sn, zn, J0{}); });
+    };
+    for (int kb = 0; kb < a.k_tiles; kb += 2) {
+      tile(kb, wcur, scur, zcur, wnxt, snxt, znxt, xr[1 & (NX - 1)], xr[2 & (NX - 1)]);
+      if (kb + 1 < a.k_tiles)
+        tile(kb + 1, wnxt, snxt, znxt, wcur, scur, zcur, xr[3 & (NX - 1)], xr[4 & (NX - 1)]);
     }
   }
 
