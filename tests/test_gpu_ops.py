@@ -195,3 +195,39 @@ def test_packed_checkpoint_to_module(tmp_path, with_zeros):
         G.assert_close_to_oracle(y.cpu().numpy(), x, o.dequantize(q, s, z, bits, 128), name)
         seen += 1
     assert seen == 2
+
+
+def test_mixnmatch_stack_through_plugin():
+    # a small Llama-shaped stack whose linears get a bitwidth each from a seeded RNG, configured
+    # the way a packed checkpoint's `layer_bitwidths` configures the plugin; every linear is
+    # checked against the oracle at its own bitwidth, at batch 1
+    import random
+
+    rnd = random.Random(0)
+    hidden, ffn, g = 256, 512, 128
+    shapes = {"self_attn.qkv_proj": (384, hidden), "self_attn.o_proj": (hidden, hidden),
+              "mlp.gate_up_proj": (2 * ffn, hidden), "mlp.down_proj": (hidden, ffn)}
+    names = [f"model.layers.{i}.{s}" for i in range(3) for s in shapes]
+    bits = {name: rnd.choice((2, 3, 4, 6, 8)) for name in names}
+    assert len(set(bits.values())) >= 4
+    cfg = vllm_matgptq.MatGPTQConfig.from_config({
+        "group_size": g, "master_bitwidth": 8, "inference_bitwidth": 4, "quant_dtype": "float16",
+        "modules_to_not_convert": ["lm_head", "norm"], "layer_bitwidths": bits})
+    for i, name in enumerate(names):
+        n, k = shapes[name.split(".", 3)[3]]
+        q, s, _ = o.make_layer(n, k, g, seed=100 + i, symmetric=True)
+        layer = vllm_matgptq.LinearBase()
+        method = cfg.get_quant_method(layer, name)
+        assert method.bitwidth == bits[name]
+        method.create_weights(layer, k, [n], k, n, torch.float16)
+        layer.qweight.data.copy_(torch.from_numpy(q))
+        layer.scales.data.copy_(torch.from_numpy(s))
+        layer.cuda()
+        method.process_weights_after_loading(layer)
+        assert layer.matgptq_weights.numel() == bits[name] * n * k // 32
+        x = o.make_activations(1, k, seed=i)
+        y = method.apply(layer, torch.from_numpy(x).cuda())
+        w = o.dequantize(q, s, np.full_like(s, 128.0), bits[name], g)
+        G.assert_close_to_oracle(y.cpu().numpy(), x, w, f"{name} b={bits[name]}")
+    assert isinstance(cfg.get_quant_method(vllm_matgptq.LinearBase(), "lm_head"),
+                      vllm_matgptq.UnquantizedLinearMethod)
