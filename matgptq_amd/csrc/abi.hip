@@ -84,17 +84,14 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     if (row_blocks >= 1024) { R = 2; S = 2; W = 4; }
     else if (row_blocks >= 320) { R = 2; }
   }
-  // default prefill tile (measured on MI355X, Llama-3-70B layers): 32 x 128 while the batch is
-  // small enough that larger tiles would leave CUs idle, 128 x 128 beyond, and 128 x 512 for
-  // the zero-point form when its workgroups fill the 256 CUs in whole rounds
+  // default prefill tile (measured on MI355X, Llama-3-70B layers): 128 x 256 (two waves per
+  // SIMD, activations copied straight into LDS) once its workgroups fill most of the 512
+  // resident slots; below that 128 x 128, and 32 x 128 while the batch is small
   if (!p->decode) {
-    if (M <= 256) {
-      p->cfg = 4;
-    } else {
-      p->cfg = 3;
-      const int64_t wgs = (N / 512) * ((M + 127) / 128);
-      if (zp && M >= 1024 && N % 512 == 0 && wgs % 256 == 0) p->cfg = 1;
-    }
+    const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
+    if (wgs_big >= 448) p->cfg = 0;
+    else if (M <= 256) p->cfg = 4;
+    else p->cfg = 3;
   }
   if (variant != 0) {
     if (variant >= 64) {

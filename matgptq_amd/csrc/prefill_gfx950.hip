@@ -6,25 +6,27 @@
 //  * a workgroup of four waves owns TM = 16*MT activation rows and 64*RBW weight
 //    rows; wave w owns the RBW row blocks [w*RBW, +RBW) of that range, so every
 //    packed code is dequantised by exactly one wave, straight from registers into
-//    the 16x32 MFMA operand, as  fp16(scale * fp16((c << (8-b)) - zero)),  the value
-//    the reference's dequantize() gives the weight;
-//  * the activation tile is staged through LDS (two buffers of 64 columns, rows padded by
-//    16 bytes so that the 16-byte operand reads of 16 rows fall into distinct banks) and
-//    shared by the four waves; global loads of a buffer are issued eight 32-column steps
-//    (four for the largest tile) before their LDS store, and every global load is branch-free (tiles beyond K or N go
-//    through a zero-length buffer descriptor), so the K loop is one straight block per step;
-//  * software pipeline inside a wave: while the matrix cores work on one 32-column step, the
-//    vector ALU dequantises the next step's weights and each activation operand register is
-//    refilled from LDS as soon as the MFMAs that read it have been issued
-//    (sched_group_barrier asks the compiler for that interleaving).  The 128 x 256 tile,
-//    whose accumulators take half of a two-waves-per-SIMD register budget, runs a lean loop
-//    without the intra-wave double buffering instead;
+//    the 16x32 MFMA operand (see dequant_pair for the arithmetic);
+//  * the 128 x 256 tile (RBW 4, MT 8: the default for large batches) runs two waves per SIMD.
+//    Its accumulators take half of a wave's 256 registers, so the activations never pass
+//    through registers: buffer_load ... lds copies them into a ring of four unpadded LDS
+//    buffers of 64 columns, three half tiles ahead, with an XOR swizzle of the 16-byte chunks
+//    against bank conflicts and hand-counted vmcnt waits in front of the workgroup barriers.
+//    One wave dequantises while the other wave of the SIMD multiplies;
+//  * the other tiles stage the activations through registers into two padded LDS buffers
+//    (global loads eight 32-column steps ahead, four for the largest tile) and pipeline inside
+//    a wave: while the matrix cores work on one 32-column step, the vector ALU dequantises the
+//    next step's weights (sched_group_barrier asks the compiler for that interleaving);
+//  * in every loop an activation operand register is refilled from LDS as soon as the MFMAs
+//    that read it have been issued, every global load is branch-free (tiles beyond K or N go
+//    through a zero-length buffer descriptor), and scales and zeros stay in registers as
+//    loaded (converted at use), so that nothing waits on a load right after issuing it;
 //  * fp32 accumulators live in registers for the whole K loop; the epilogue packs
 //    four consecutive output columns per lane into one 8-byte store.
 //
 // Measured on this target: a loop of nothing but independent MFMAs reaches 1.37 PFLOP/s with
-// one wave per SIMD and 1.91 PFLOP/s with two (nominal 2.5), which is why tiles are sized
-// for two resident waves per SIMD.
+// one wave per SIMD and 1.91 PFLOP/s with two (nominal 2.5), which is why the default tile is
+// sized for two resident waves per SIMD.
 //
 // Workgroup ids are remapped so that the workgroups of one XCD (ids congruent
 // modulo 8) walk consecutive activation tiles of the same weight rows and share
@@ -46,22 +48,29 @@ constexpr int kXs = 64;          // activation columns per LDS stage
 #endif
 constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 
-// One raw pair -> two weights.  u = c - 2^(b-1) is exact; with a zero point
-// v = m*u - (zero - 128) = (c << (8-b)) - zero is rounded once (exact for integral
-// zeros) and multiplied by the scale; without, `scale` already carries the factor
-// m = 2^(8-b) (a power of two, so the single rounding of the product is unchanged).
-// bf16 storage: a bf16 scale can lie far below fp16's normal range, so the caller passes
-// scale * 2^8 (and zrel * 2^-8) and v is formed as v * 2^-8, exact as well; the
-// symmetric form takes the same route with zrel = 0.
+// One raw pair -> two weights.  u = c - 2^(b-1) is exact.
+//   symmetric, fp16 storage:  w = u * (scale * m),  m = 2^(8-b) (a power of two: one rounding,
+//     the value the reference's dequantize() gives);
+//   zero point, fp16 storage: w = fma(u, scale * m, -(scale * zrel)),  zrel = zero - 128: two
+//     instructions per pair instead of three.  scale * zrel is rounded to fp16 before the fma,
+//     so w can differ from dequantize()'s  fp16(scale * fp16(m u - zrel))  by one rounding of a
+//     term no larger than 128 scale: at most scale / 16, less than the rounding error of w
+//     itself (the dense dequantize_matgptq operator keeps the reference's exact sequence);
+//   bf16 storage: a bf16 scale can lie far below fp16's normal range, so the caller passes
+//     scale * 2^8 and zrel * 2^-8 and  v = m u 2^-8 - zrel 2^-8  is formed exactly and
+//     multiplied by the scale (the symmetric form takes the same route with zrel = 0).
+// `a`, `b`: (scale * m, scale * zrel) for fp16 storage with zero points, (scale', zrel') else.
 template <int BITS, int P, bool ZP>
-__device__ __forceinline__ half2v dequant_pair(uint32_t raw, half2v zrel, half2v scale) {
+__device__ __forceinline__ half2v dequant_pair(uint32_t raw, half2v b, half2v a) {
   const half2v u = centre_raw<P>(raw, Codec<BITS>::kCentre);
-  if constexpr (ZP || kBf16) {
-    constexpr float m = (float)(1 << (8 - BITS)) * (kBf16 ? 1.0f / 256.0f : 1.0f);
-    const half2v v = __builtin_elementwise_fma(u, h2_splat(m), -zrel);
-    return v * scale;
+  if constexpr (kBf16) {
+    constexpr float m = (float)(1 << (8 - BITS)) / 256.0f;
+    const half2v v = __builtin_elementwise_fma(u, h2_splat(m), -b);
+    return v * a;
+  } else if constexpr (ZP) {
+    return __builtin_elementwise_fma(u, a, -b);
   } else {
-    return u * scale;
+    return u * a;
   }
 }
 
@@ -77,10 +86,10 @@ __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const U
 }
 
 // Two waves per SIMD (256 registers each) whenever the accumulators leave room for the rest:
-// one wave alone cannot keep the matrix pipe busy.  A tile whose accumulators take half of
-// that budget runs the lean loop below (no intra-wave double buffering).
-constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 <= 128 ? 2 : 1; }
-constexpr bool prefill_lean(int rbw, int mt) { return rbw * mt * 4 == 128; }
+// one wave alone cannot keep the matrix pipe busy.  The tile whose accumulators take half of
+// that budget runs the ring loop below (activations straight into LDS, one operand set).
+constexpr bool prefill_lean(int rbw, int mt) { return rbw == 4 && mt == 8; }
+constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
 template <int BITS, int GROUP, bool ZP, int RBW, int MT>
 __global__ void __launch_bounds__(256, prefill_min_waves(RBW, MT))
@@ -89,7 +98,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   constexpr int GPT = GROUP == 32 ? 4 : 1;
   constexpr int XCHUNKS = TM * (kXs / 8) / 256;  // 16-byte chunks per thread per stage
   static_assert(TM * (kXs / 8) % 256 == 0, "activation tile must split evenly over 256 threads");
-  __shared__ __align__(16) _Float16 xs[2][TM * kXsPitch];
+  __shared__ __align__(16) _Float16 xs[2][prefill_lean(RBW, MT) ? 8 : TM * kXsPitch];  // (unused by the ring loop)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -119,12 +128,14 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 
   const UnpackConsts<BITS> kc_unpack;
   uint32_t wcur[RBW][BITS], wnxt[RBW][BITS];
-  _Float16 scur[RBW][GPT], snxt[RBW][GPT];
-  _Float16 zcur[RBW][GPT], znxt[RBW][GPT];
+  // scales and zeros as loaded (16 bits in a register each): converted where they are used, so
+  // that nothing has to wait for these loads right after they are issued
+  uint32_t scur[RBW][GPT], snxt[RBW][GPT];
+  uint32_t zcur[RBW][GPT], znxt[RBW][GPT];
 
   // Branch-free loads: a tile beyond K, or a row block beyond N, is read through a
   // descriptor of zero length (every lane out of range: zeros come back, nothing is fetched).
-  auto load_weights = [&](uint32_t (&w)[RBW][BITS], _Float16 (&s)[RBW][GPT], _Float16 (&z)[RBW][GPT],
+  auto load_weights = [&](uint32_t (&w)[RBW][BITS], uint32_t (&s)[RBW][GPT], uint32_t (&z)[RBW][GPT],
                           int kb) {
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
@@ -142,23 +153,9 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
       for (int gg = 0; gg < GPT; gg++) {
         const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
         const uint32_t so = ((uint32_t)rb * a.G + g) * 32;  // bytes
-        // fp16: the scale as stored (times 2^(8-b) in the symmetric form, applied below) and
-        // zero - 128; bf16: scale * 2^8 and (zero - 128) * 2^-8, converted through fp32
-        const uint16_t sbits = __builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0);
-        if constexpr (kBf16) {
-          s[rr][gg] = (_Float16)(bf16_bits_to_float(sbits) * 256.0f);
-        } else {
-          s[rr][gg] = __builtin_bit_cast(_Float16, sbits);
-        }
-        if constexpr (ZP) {
-          const uint16_t zbits = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
-          if constexpr (kBf16)
-            z[rr][gg] = (_Float16)((bf16_bits_to_float(zbits) - 128.0f) * (1.0f / 256.0f));
-          else
-            z[rr][gg] = __builtin_bit_cast(_Float16, zbits) - (_Float16)128.0f;
-        } else {
-          z[rr][gg] = (_Float16)0.0f;
-        }
+        s[rr][gg] = __builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0);
+        if constexpr (ZP) z[rr][gg] = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
+        else z[rr][gg] = 0u;
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -176,7 +173,6 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     x_voff[c] = m < (uint32_t)a.M ? (m * (uint32_t)a.K + col8 * 8) * 2u : x_bytes;
     x_lds[c] = (uint32_t)(row * kXsPitch + col8 * 8);
   }
-  u32x4 xa[XCHUNKS];  // the lean loop's single set
   auto load_x = [&](u32x4 (&xr)[XCHUNKS], int h) {  // columns [h*64, +64)
 #ifdef MATGPTQ_DEBUG_NOXLOAD
     const bool valid = h < 0;
@@ -195,17 +191,25 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
       *reinterpret_cast<half8*>(&xs[buf][x_lds[c]]) = storage8_to_half8(__builtin_bit_cast(half8, xr[c]));
   };
 
-  auto dequant_step = [&](Frag (&aw)[RBW], const uint32_t (&w)[RBW][BITS], const _Float16 (&s)[RBW][GPT],
-                          const _Float16 (&z)[RBW][GPT], auto jtag) {
+  auto dequant_step = [&](Frag (&aw)[RBW], const uint32_t (&w)[RBW][BITS], const uint32_t (&s)[RBW][GPT],
+                          const uint32_t (&z)[RBW][GPT], auto jtag) {
     constexpr int J = decltype(jtag)::value;
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
       const int gg = GROUP == 32 ? J : 0;
-      _Float16 s1 = s[rr][gg];
-      if constexpr (!ZP && !kBf16) s1 = (_Float16)((float)s1 * (float)(1 << (8 - BITS)));
+      // fp16 storage: scale * 2^(8-b) and scale * (zero - 128);
+      // bf16 storage: scale * 2^8 and (zero - 128) * 2^-8, converted through fp32
+      _Float16 s1, z1 = (_Float16)0.f;
+      if constexpr (kBf16) {
+        s1 = (_Float16)(bf16_bits_to_float(s[rr][gg]) * 256.0f);
+        if constexpr (ZP) z1 = (_Float16)((bf16_bits_to_float(z[rr][gg]) - 128.0f) * (1.0f / 256.0f));
+      } else {
+        const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)s[rr][gg]);
+        s1 = (_Float16)((float)s0 * (float)(1 << (8 - BITS)));  // scale * m
+        if constexpr (ZP) z1 = s0 * (__builtin_bit_cast(_Float16, (uint16_t)z[rr][gg]) - (_Float16)128.0f);
+      }
       const half2v sc = {s1, s1};
-      half2v zr = {(_Float16)0.f, (_Float16)0.f};
-      if constexpr (ZP) zr = half2v{z[rr][gg], z[rr][gg]};
+      const half2v zr = {z1, z1};
 #ifdef MATGPTQ_DEBUG_NODEQUANT
       aw[rr].u[0] = w[rr][0]; aw[rr].u[1] = w[rr][1 % BITS]; aw[rr].u[2] = w[rr][0] ^ J; aw[rr].u[3] = w[rr][1 % BITS];
       (void)sc; (void)zr;
@@ -245,43 +249,108 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   };
 
   if constexpr (prefill_lean(RBW, MT)) {
-    // Lean loop: one operand set, weights reloaded in place as soon as their last octet is
-    // dequantised; the other wave of the SIMD covers the latencies.
-    Frag aw[RBW];
-    auto lean_step = [&](int buf, int jj, auto jtag, auto&& after_dequant) {
-      dequant_step(aw, wcur, scur, zcur, jtag);
-      after_dequant();
-      constexpr int MG = 2;
+    // The 128 x 256 tile at two waves per SIMD: its accumulators take half of the wave's 256
+    // registers, so the activations never pass through registers.  buffer_load ... lds copies
+    // them from global memory straight into a ring of four LDS buffers (one half tile of 64
+    // columns each, 128 rows of 128 bytes, no padding), three half tiles ahead of their use.
+    // A wave copies 8 rows per instruction (lane l: row l/8, 16-byte chunk l%8 of the LDS
+    // row); chunk c of LDS row r holds columns 8*(c ^ ((r>>1)&7)) of the half tile, so the
+    // sixteen lanes of an operand read (rows r..r+15, one column chunk) hit sixteen different
+    // 16-byte bank groups.  The waits for these copies are written by hand: vmcnt counts every
+    // buffer load of the wave in issue order, and each wait below names how many younger ones
+    // may still be in flight (see the issue order at the loop).
+    __shared__ __align__(16) _Float16 ring0[TM * kXs];
+    __shared__ __align__(16) _Float16 ring1[TM * kXs];
+    __shared__ __align__(16) _Float16 ring2[TM * kXs];
+    __shared__ __align__(16) _Float16 ring3[TM * kXs];
+    static_assert(TM == 128, "the copy below moves 32 rows per wave");
+    // this lane's part of a copy: rows wave*32 + i*8 + lane/8, LDS chunk lane%8
+    uint32_t dma_voff[4];
 #pragma unroll
-      for (int m0g = 0; m0g < MT; m0g += MG) {
-        Frag b[MG];
+    for (int i = 0; i < 4; i++) {
+      const int r = wave * 32 + i * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ ((r >> 1) & 7);
+      const uint32_t m = (uint32_t)(m0 + r);
+      dma_voff[i] = m < (uint32_t)a.M ? (m * (uint32_t)a.K + c * 8) * 2u : x_bytes;
+    }
+    auto dma = [&](_Float16* ring, int ih) {  // half tile ih of the walk into `ring`
+      const bool valid = ih < 2 * a.k_tiles;
+      const BufRsrc xres = make_rsrc(a.x, valid ? x_bytes : 0u);
 #pragma unroll
-        for (int i = 0; i < MG; i++) read_frag(b[i], m0g + i, buf, jj);
-#pragma unroll
-        for (int i = 0; i < MG; i++) {
-#pragma unroll
-          for (int rr = 0; rr < RBW; rr++)
-            acc[rr][m0g + i] =
-                __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b[i].h, acc[rr][m0g + i], 0, 0, 0);
-        }
-      }
+      for (int i = 0; i < 4; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            xres, (__attribute__((address_space(3))) void*)(ring + (wave * 32 + i * 8) * kXs), 16, dma_voff[i],
+            (uint32_t)ih * (kXs * 2), 0, 0);
     };
-    auto nothing = [] {};
-    load_x(xa, 0);
+    // operand read: row i*16 + r16, columns [jj*32 + q*8, +8)
+    const int sw = (r16 >> 1) & 7;
+    const int frag_off[2] = {r16 * kXs + ((q ^ sw) * 8), r16 * kXs + (((4 + q) ^ sw) * 8)};
+    auto ring_frag = [&](Frag& bv, const _Float16* ring, int i, int jj) {
+      bv.v = *reinterpret_cast<const uint4*>(ring + i * 16 * kXs + frag_off[jj]);
+    };
+    // wait until at most `n` buffer loads of this wave are in flight, then meet the workgroup
+    auto wait_and_meet = [&](auto ntag) {
+      // (the counter holds 63 at most: with more younger loads than that, 63 still excludes the
+      // one waited for)
+      constexpr int n = decltype(ntag)::value < 63 ? decltype(ntag)::value : 63;
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt((n & 15) | (7 << 4) | (0 << 8) | ((n >> 4) << 14));  // vmcnt(n), lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // one 32-column step: dequantise octet J of the tile into `aw`, multiply by the operands in
+    // `bv`, and refill each bv[i] for the next step (ring `nring`, columns [njj*32, +32)) as soon
+    // as its MFMAs are issued.  Two waves share a SIMD: one's vector work overlaps the other's
+    // matrix work, which is why a single operand set is enough.
+    Frag aw[RBW];
+    Frag bv[MT];
+    auto dstep = [&](const uint32_t (&w)[RBW][BITS], const uint32_t (&sv)[RBW][GPT], const uint32_t (&zv)[RBW][GPT],
+                     auto jtag, const _Float16* nring, int njj) {
+      dequant_step(aw, w, sv, zv, jtag);
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+#pragma unroll
+        for (int rr = 0; rr < RBW; rr++)
+          acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, bv[i].h, acc[rr][i], 0, 0, 0);
+        ring_frag(bv[i], nring, i, njj);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using J0 = std::integral_constant<int, 0>;
+    using J1 = std::integral_constant<int, 1>;
+    using J2 = std::integral_constant<int, 2>;
+    using J3 = std::integral_constant<int, 3>;
+    constexpr int kW = RBW * (BITS == 3 || BITS == 6 || BITS == 8 ? 2 : 1) + RBW * GPT * (ZP ? 2 : 1);  // buffer loads of load_weights
+    // issue order of the wave's buffer loads: prologue  D0 D1 D2 D3 W0 W1 ; then per tile t
+    //   after the first barrier D(2t+4), after the second barrier D(2t+5), at its end W(t+2)
+    // (D = 4 copies of one half tile, W = kW loads of one tile's codes, scales and zeros)
+    dma(ring0, 0);
+    dma(ring1, 1);
+    dma(ring2, 2);
+    dma(ring3, 3);
     load_weights(wcur, scur, zcur, 0);
-    store_x(xa, 0);
-    __syncthreads();
-    for (int kb = 0; kb < a.k_tiles; kb++) {
-      load_x(xa, 2 * kb + 1);
-      lean_step(0, 0, std::integral_constant<int, 0>{}, nothing);
-      lean_step(0, 1, std::integral_constant<int, 1>{}, nothing);
-      store_x(xa, 1);
-      __syncthreads();
-      load_x(xa, 2 * kb + 2);
-      lean_step(1, 0, std::integral_constant<int, 2>{}, nothing);
-      lean_step(1, 1, std::integral_constant<int, 3>{}, [&] { load_weights(wcur, scur, zcur, kb + 1); });
-      store_x(xa, 0);
-      __syncthreads();
+    load_weights(wnxt, snxt, znxt, 1);
+    wait_and_meet(std::integral_constant<int, 12 + 2 * kW>{});  // D0 has landed
+#pragma unroll
+    for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
+    // one tile; ra / rb: the rings of its two half tiles, rn: the ring of the next tile's first
+    auto dtile = [&](int kb, uint32_t (&wc)[RBW][BITS], uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT],
+                     _Float16* ra, _Float16* rb, _Float16* rn) {
+      dstep(wc, sc, zc, J0{}, ra, 1);
+      // needs D(2kb+1); younger in steady state: W(kb) D(2kb+2) D(2kb+3) W(kb+1)
+      wait_and_meet(std::integral_constant<int, 8 + 2 * kW>{});
+      dma(ra, 2 * kb + 4);  // every wave is past its reads of ra
+      dstep(wc, sc, zc, J1{}, rb, 0);
+      dstep(wc, sc, zc, J2{}, rb, 1);
+      // needs D(2kb+2); younger: D(2kb+3) W(kb+1) D(2kb+4)
+      wait_and_meet(std::integral_constant<int, 8 + kW>{});
+      dma(rb, 2 * kb + 5);
+      dstep(wc, sc, zc, J3{}, rn, 0);
+      load_weights(wc, sc, zc, kb + 2);  // this set is free now
+    };
+    for (int kb = 0; kb < a.k_tiles; kb += 2) {
+      dtile(kb, wcur, scur, zcur, ring0, ring1, ring2);
+      if (kb + 1 < a.k_tiles) dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
     }
   } else {
   Frag awA[RBW], awB[RBW];
@@ -347,9 +416,9 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 
     // one tile: weights `wc` (the next tile's are in `wn`), activation sets `sa` / `sb` for
     // the half tiles 2 kb + 1 (LDS buffer 1) and 2 kb + 2 (buffer 0)
-    auto tile = [&](int kb, uint32_t (&wc)[RBW][BITS], _Float16 (&sc)[RBW][GPT], _Float16 (&zc)[RBW][GPT],
-                    const uint32_t (&wn)[RBW][BITS], const _Float16 (&sn)[RBW][GPT],
-                    const _Float16 (&zn)[RBW][GPT], u32x4 (&sa)[XCHUNKS], u32x4 (&sb)[XCHUNKS]) {
+    auto tile = [&](int kb, uint32_t (&wc)[RBW][BITS], uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT],
+                    const uint32_t (&wn)[RBW][BITS], const uint32_t (&sn)[RBW][GPT],
+                    const uint32_t (&zn)[RBW][GPT], u32x4 (&sa)[XCHUNKS], u32x4 (&sb)[XCHUNKS]) {
       step(awA, bf, 0, 1, [&] { dequant_step(awB, wc, sc, zc, J1{}); });
       store_x(sa, 1);  // buffer 1 was last read during step 2 of the previous tile
       load_x(sa, 2 * kb + 1 + NX);
