@@ -223,6 +223,10 @@ __device__ __forceinline__ BufRsrc make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
+// Number of load instructions load_tile_words issues for one tile (kernels that count their
+// loads in flight by hand use it).
+constexpr int tile_load_count(int bits) { return bits == 3 || bits == 6 || bits == 8 ? 2 : 1; }
+
 // Loads the BITS words of `lane` from the tile that starts `tile_bytes` into the buffer
 // (wave-uniform), one load per segment.  AUX = kAuxStream for data read once (decode),
 // 0 for data other workgroups read again (prefill).

@@ -320,7 +320,8 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     using J1 = std::integral_constant<int, 1>;
     using J2 = std::integral_constant<int, 2>;
     using J3 = std::integral_constant<int, 3>;
-    constexpr int kW = RBW * (BITS == 3 || BITS == 6 || BITS == 8 ? 2 : 1) + RBW * GPT * (ZP ? 2 : 1);  // buffer loads of load_weights
+    // buffer loads one load_weights() issues: the codes, then a scale (and a zero) per group
+    constexpr int kW = RBW * tile_load_count(BITS) + RBW * GPT * (ZP ? 2 : 1);
     // issue order of the wave's buffer loads: prologue  D0 D1 D2 D3 W0 W1 ; then per tile t
     //   after the first barrier D(2t+4), after the second barrier D(2t+5), at its end W(t+2)
     // (D = 4 copies of one half tile, W = kW loads of one tile's codes, scales and zeros)

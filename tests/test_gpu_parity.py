@@ -112,6 +112,22 @@ def _decode_variants():
     return [1 | (v << 8) | (flavour << 16) for v in range(1, 43) for flavour in (1, 2)]
 
 
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_prefill_ring_tile_every_format(b, g, zp):
+    # the 128 x 256 tile counts its loads in flight by hand, and the count depends on the
+    # bitwidth (one or two code segments), the group size and the zero points; ragged M and N,
+    # odd number of K tiles
+    n, k, m = 304, 128 * 7, 200
+    lay = G.Layer(n, k, b, g, seed=31 * b + (g & 7), zero_points=zp)
+    x = o.make_activations(m, k, seed=b)
+    for _ in range(2):
+        y = lay.run(x, flags=1 | (64 << 8))
+        G.assert_close_to_oracle(y, x, lay.w, f"ring tile b={b} g={g} zp={zp}")
+    assert _lib.describe_plan(b, g, n, k, m, zp, 1 | (64 << 8)).endswith("cfg0")
+
+
 def test_decode_every_work_split():
     # all (R, S, W) shapes in both flavours; 65 row blocks leave idle slots in the last
     # workgroup, K = 4096 gives up to 32 tiles per wave
