@@ -89,7 +89,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   // resident slots; below that 128 x 128, and 32 x 128 while the batch is small
   if (!p->decode) {
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
-    if (wgs_big >= 448) p->cfg = 0;
+    // (bf16 storage has no ring loop: its 128 x 256 tile runs one wave per SIMD)
+    if (wgs_big >= 448 && !(flags & MATGPTQ_FLAG_BF16)) p->cfg = 0;
     else if (M <= 256) p->cfg = 4;
     else p->cfg = 3;
   }

@@ -88,7 +88,9 @@ __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const U
 // Two waves per SIMD (256 registers each) whenever the accumulators leave room for the rest:
 // one wave alone cannot keep the matrix pipe busy.  The tile whose accumulators take half of
 // that budget runs the ring loop below (activations straight into LDS, one operand set).
-constexpr bool prefill_lean(int rbw, int mt) { return rbw == 4 && mt == 8; }
+// (bf16 storage: the copy into LDS would bypass the bf16 -> fp16 conversion, so that build keeps
+// the staged loop for this tile as well)
+constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && rbw == 4 && mt == 8; }
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
 template <int BITS, int GROUP, bool ZP, int RBW, int MT>

@@ -319,3 +319,19 @@ def test_reference_kernel_test_grid_bf16(b, k, m, gsz):
     pk = G.pack_device(codes, b, from_master=False)
     y = _gemm_bf16(b, gsz, n, k, x, pk, scales, None)
     assert np.array_equal(y.view(np.uint32), expect.view(np.uint32))
+
+
+@pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8)))
+def test_bf16_prefill_large_tiles(flags):
+    # default choice for a large batch, and the two largest tiles forced
+    n, k, m, b, g = 2048, 1024, 2048, 4, 128
+    q, s16, z16 = o.make_layer(n, k, g, seed=77)
+    s = o.round_to_bf16(s16.astype(np.float32))
+    z = z16.astype(np.float32)
+    x = o.round_to_bf16(o.make_activations(m, k, seed=8).astype(np.float32))
+    pk = G.pack_device(q, b, True)
+    y = _gemm_bf16(b, g, n, k, x, pk, s, z, flags=flags)
+    rows = np.r_[0:64, m - 64:m]
+    ref = o.linear_f64(x[rows], o.dequantize_bf16(q, s, z, b, g))
+    assert np.all(np.isfinite(y))
+    assert np.max(np.abs(y[rows] - ref)) <= G.REL_TOL * np.max(np.abs(ref))
