@@ -313,12 +313,33 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     auto dstep = [&](const uint32_t (&w)[RBW][BITS], const uint32_t (&sv)[RBW][GPT], const uint32_t (&zv)[RBW][GPT],
                      auto jtag, const _Float16* nring, int njj) {
       dequant_step(aw, w, sv, zv, jtag);
+      // two halves of two row blocks each: the vector work of the second half can be issued
+      // between the MFMAs of the first; the operands are refilled behind the second half
 #pragma unroll
       for (int i = 0; i < MT; i++) {
 #pragma unroll
-        for (int rr = 0; rr < RBW; rr++)
+        for (int rr = 0; rr < RBW / 2; rr++)
+          acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, bv[i].h, acc[rr][i], 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+#pragma unroll
+        for (int rr = RBW / 2; rr < RBW; rr++)
           acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, bv[i].h, acc[rr][i], 0, 0, 0);
         ring_frag(bv[i], nring, i, njj);
+      }
+      constexpr int kHalf = (RBW / 2) * MT;           // MFMAs per half
+      constexpr int kValuHalf = (RBW / 2) * 26;       // vector instructions of two row blocks, roughly
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuHalf, 0);
+#pragma unroll
+      for (int n = 0; n < kHalf; n++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (kValuHalf + kHalf - 1) / kHalf, 0);
+      }
+#pragma unroll
+      for (int n = 0; n < kHalf; n++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (n & 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
