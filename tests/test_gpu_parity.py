@@ -335,3 +335,24 @@ def test_bf16_prefill_large_tiles(flags):
     ref = o.linear_f64(x[rows], o.dequantize_bf16(q, s, z, b, g))
     assert np.all(np.isfinite(y))
     assert np.max(np.abs(y[rows] - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("b,g,zp", [(4, 128, True), (3, 32, True), (8, 128, False), (2, -1, True), (6, 128, True)])
+def test_prefill_tiles_agree_bit_for_bit(b, g, zp):
+    # every tile accumulates the same products in the same order, so two tiles must give the same
+    # bits; the ring tile (hand-counted waits, asynchronous copies into LDS) is compared with a
+    # staged tile on a problem large enough to keep every CU busy for several rounds
+    n, k, m = 4096, 2048, 2048
+    rng = np.random.default_rng(b)
+    packed = torch.from_numpy(rng.integers(-2 ** 31, 2 ** 31, _lib.load().matgptq_packed_words(b, n, k),
+                                           dtype=np.int64).astype(np.int32)).to(G.DEV)
+    groups = n * (1 if g == -1 else k // g)
+    scales = torch.from_numpy((rng.random(groups) * 0.01 + 1e-3).astype(np.float16)).to(G.DEV)
+    zeros = torch.from_numpy(rng.integers(0, 256, groups).astype(np.float16)).to(G.DEV) if zp else None
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float16)).to(G.DEV)
+    ring = [G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (64 << 8)).clone() for _ in range(3)]
+    staged = G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (67 << 8))
+    torch.cuda.synchronize()
+    assert torch.isfinite(staged.float()).all()
+    for y in ring:
+        assert torch.equal(y, staged)
