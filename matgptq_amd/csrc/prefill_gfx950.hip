@@ -7,8 +7,9 @@
 //    rows; wave w owns the RBW row blocks [w*RBW, +RBW) of that range, so every
 //    packed code is dequantised by exactly one wave, straight from registers into
 //    the 16x32 MFMA operand (see dequant_pair for the arithmetic);
-//  * the 128 x 256 tile (RBW 4, MT 8: the default for large batches) runs two waves per SIMD.
-//    Its accumulators take half of a wave's 256 registers, so the activations never pass
+//  * the 128 x 256 tile (RBW 4, MT 8: the default for large batches) and the 128 x 128 tile
+//    (RBW 2, MT 8) run two waves per SIMD with a ring loop.  The accumulators of the larger one
+//    take half of a wave's 256 registers, so the activations never pass
 //    through registers: buffer_load ... lds copies them into a ring of four unpadded LDS
 //    buffers of 64 columns, three half tiles ahead, with an XOR swizzle of the 16-byte chunks
 //    against bank conflicts and hand-counted vmcnt waits in front of the workgroup barriers.
@@ -90,7 +91,7 @@ __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const U
 // that budget runs the ring loop below (activations straight into LDS, one operand set).
 // (bf16 storage: the copy into LDS would bypass the bf16 -> fp16 conversion, so that build keeps
 // the staged loop for this tile as well)
-constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && rbw == 4 && mt == 8; }
+constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && (rbw == 4 || rbw == 2) && mt == 8; }
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
 template <int BITS, int GROUP, bool ZP, int RBW, int MT>

@@ -351,7 +351,8 @@ def test_prefill_tiles_agree_bit_for_bit(b, g, zp):
     zeros = torch.from_numpy(rng.integers(0, 256, groups).astype(np.float16)).to(G.DEV) if zp else None
     x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float16)).to(G.DEV)
     ring = [G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (64 << 8)).clone() for _ in range(3)]
-    staged = G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (67 << 8))
+    ring.append(G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (67 << 8)).clone())  # 128 x 128 ring tile
+    staged = G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (66 << 8))  # 64 x 256, staged
     torch.cuda.synchronize()
     assert torch.isfinite(staged.float()).all()
     for y in ring:
