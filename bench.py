@@ -256,6 +256,12 @@ def main() -> int:
             "weight_GBps": round(total_bytes / t / 1e9, 1)}
         del stack
         torch.cuda.empty_cache()
+        # ------------------------ the same decoder end to end (configs[3]): tokens/s
+        # linears through the module, norms / rotary / attention over a static cache at context
+        # 512 / dense head / argmax as torch operators, one token per HIP graph replay
+        from matgptq_amd import decoder
+        extra["mixnmatch_decoder_end_to_end"] = decoder.measure(layers=32, context=512, new_tokens=64)
+        torch.cuda.empty_cache()
         # --------------------------------------------------------------- prefill
         pre = {}
         m = 2048

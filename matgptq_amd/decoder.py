@@ -1,0 +1,345 @@
+"""Callers of the bit-sliced linear: a Llama-shaped decoder whose linears are `MatGPTQLinear`
+modules at per-layer bitwidths (Mix'n'Match), with a static key/value cache and a decode step
+that can be captured into a HIP graph.
+
+Counterpart of the reference's transformers path:
+  replace_with_matgptq_linear   inference_lib/inference_demo_transformers.py:17-56 (same name and
+                                arguments; works on any `torch.nn.Module` tree, so also on a
+                                transformers model)
+  DecodeSession.generate        inference_lib/inference_demo_transformers.py:134-176
+  DecodeSession.tokens_per_s    inference_lib/bench_transformers_e2e.py:61-76,160-166
+
+The reference wraps the step in `torch.compile(mode="reduce-overhead")` to get a device graph;
+here the step is written with device-side position and token tensors and captured directly
+(`torch.cuda.CUDAGraph` is a HIP graph on ROCm).  Only the linears are the product: norms,
+rotary embedding, attention and the head are plain torch operators.
+
+    python -m matgptq_amd.decoder [--layers 32] [--context 512] [--new_tokens 64] [--bits 2 3 4 6 8]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import time
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from .checkpoint import load_quantised_layer, read_layer_bitwidths
+from .ops import matryoshka_slice
+
+
+def replace_with_matgptq_linear(model: torch.nn.Module, quantized_weights_path: Union[str, os.PathLike],
+                                quantized_config_path: Optional[str] = None, master_bitwidth: int = 8,
+                                slice_bitwidth: int = 8, group_size: int = 128) -> torch.nn.Module:
+    """Replaces submodules of `model` by `MatGPTQLinear` modules built from the quantiser's
+    per-layer directories `<quantized_weights_path>/<dotted.layer.name>/data.pt`.
+
+    With `quantized_config_path` (lines `layer_name: bitwidth`, as written by the reference's
+    search, evo_quant_search.py:660-672) exactly the listed layers are replaced, each at its own
+    bitwidth; without it every layer directory is replaced at `slice_bitwidth`.  A stored
+    `zero` tensor is used when present (the reference drops it and assumes 128).
+    """
+    from matgptq_cuda.matgptq_linear import MatGPTQLinear
+
+    def _replace(layer_name: str, bitwidth: int) -> None:
+        data = load_quantised_layer(os.path.join(quantized_weights_path, layer_name))
+        codes = matryoshka_slice(data["qweight"].cuda(), master_bitwidth, bitwidth)
+        zero = data.get("zero")
+        layer = MatGPTQLinear(codes, data["scale"].cuda(), bitwidth, group_size,
+                              zeros=zero.cuda() if zero is not None else None)
+        *parent_path, attr = layer_name.split(".")
+        parent = model.get_submodule(".".join(parent_path)) if parent_path else model
+        setattr(parent, attr, layer)
+
+    if quantized_config_path:
+        for layer_name, bitwidth in read_layer_bitwidths(quantized_config_path).items():
+            _replace(layer_name, bitwidth)
+    else:
+        for layer_name in sorted(os.listdir(quantized_weights_path)):
+            if os.path.isdir(os.path.join(quantized_weights_path, layer_name)):
+                _replace(layer_name, slice_bitwidth)
+    return model
+
+
+@dataclass
+class DecoderConfig:
+    """Shape of the decoder; the defaults are Llama-3-8B's."""
+    hidden: int = 4096
+    ffn: int = 14336
+    layers: int = 32
+    heads: int = 32
+    kv_heads: int = 8
+    vocab: int = 128256
+    rope_theta: float = 500000.0
+    rms_eps: float = 1e-5
+    group_size: int = 128
+
+    @property
+    def head_dim(self) -> int:
+        return self.hidden // self.heads
+
+    def linear_shapes(self) -> Dict[str, tuple]:
+        """`name -> (N, K)` of the four linears of a block (q, k, v fused; gate, up fused)."""
+        return {"qkv": ((self.heads + 2 * self.kv_heads) * self.head_dim, self.hidden),
+                "o": (self.hidden, self.hidden),
+                "gate_up": (2 * self.ffn, self.hidden),
+                "down": (self.hidden, self.ffn)}
+
+
+class Block(torch.nn.Module):
+    """One decoder block.  The linears may be any module mapping `[M, K] -> [M, N]`."""
+
+    def __init__(self, cfg: DecoderConfig, linears: Dict[str, torch.nn.Module], dtype, device):
+        super().__init__()
+        self.cfg = cfg
+        self.qkv, self.o = linears["qkv"], linears["o"]
+        self.gate_up, self.down = linears["gate_up"], linears["down"]
+        self.input_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=dtype, device=device), requires_grad=False)
+        self.post_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=dtype, device=device), requires_grad=False)
+
+    def forward(self, h, cos, sin, pos, k_cache, v_cache, mask):
+        """h [M, hidden]; cos/sin [M, head_dim]; pos int64 [M] (cache rows written);
+        k_cache/v_cache [kv_heads, ctx, head_dim]; mask bool [M, ctx] (True = attend)."""
+        cfg = self.cfg
+        m, d, rep = h.shape[0], cfg.head_dim, cfg.heads // cfg.kv_heads
+        x = torch.nn.functional.rms_norm(h, (cfg.hidden,), self.input_norm, cfg.rms_eps)
+        qkv = self.qkv(x).view(m, cfg.heads + 2 * cfg.kv_heads, d)
+        q, k, v = qkv[:, :cfg.heads], qkv[:, cfg.heads:cfg.heads + cfg.kv_heads], qkv[:, cfg.heads + cfg.kv_heads:]
+        q, k = _rotate(q, cos, sin), _rotate(k, cos, sin)
+        k_cache.index_copy_(1, pos, k.transpose(0, 1))
+        v_cache.index_copy_(1, pos, v.transpose(0, 1))
+        # grouped-query attention: the `rep` query heads of a key/value head share one batched product
+        qg = q.transpose(0, 1).reshape(cfg.kv_heads, rep * m, d)
+        scores = torch.bmm(qg, k_cache.transpose(1, 2)).float() * (d ** -0.5)  # [kv, rep*m, ctx]
+        scores = scores.view(cfg.kv_heads, rep, m, -1).masked_fill(~mask, float("-inf"))
+        probs = torch.softmax(scores, dim=-1).to(h.dtype).view(cfg.kv_heads, rep * m, -1)
+        attn = torch.bmm(probs, v_cache).view(cfg.heads, m, d).transpose(0, 1).reshape(m, cfg.hidden)
+        h = h + self.o(attn)
+        x = torch.nn.functional.rms_norm(h, (cfg.hidden,), self.post_norm, cfg.rms_eps)
+        gu = self.gate_up(x)
+        h = h + self.down(torch.nn.functional.silu(gu[:, :cfg.ffn]) * gu[:, cfg.ffn:])
+        return h
+
+
+def _rotate(t, cos, sin):
+    """Rotary embedding, half-split convention: t [M, heads, d], cos/sin [M, d]."""
+    half = t.shape[-1] // 2
+    rot = torch.cat((-t[..., half:], t[..., :half]), dim=-1)
+    return t * cos[:, None, :] + rot * sin[:, None, :]
+
+
+class Decoder(torch.nn.Module):
+    def __init__(self, cfg: DecoderConfig, blocks: Sequence[Block], embed: torch.Tensor, head: torch.Tensor,
+                 max_context: int):
+        super().__init__()
+        self.cfg = cfg
+        self.blocks = torch.nn.ModuleList(blocks)
+        self.embed = torch.nn.Parameter(embed, requires_grad=False)     # [vocab, hidden]
+        self.head = torch.nn.Parameter(head, requires_grad=False)       # [vocab, hidden], dense like the reference's lm_head
+        self.final_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=embed.dtype, device=embed.device),
+                                             requires_grad=False)
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, dtype=torch.float32) / cfg.head_dim))
+        ang = torch.outer(torch.arange(max_context, dtype=torch.float32), inv)
+        ang = torch.cat((ang, ang), dim=-1)
+        self.register_buffer("cos", ang.cos().to(embed.dtype).to(embed.device), persistent=False)
+        self.register_buffer("sin", ang.sin().to(embed.dtype).to(embed.device), persistent=False)
+        self.register_buffer("arange", torch.arange(max_context, device=embed.device), persistent=False)
+        self.max_context = max_context
+
+    def new_cache(self):
+        cfg = self.cfg
+        shape = (len(self.blocks), 2, cfg.kv_heads, self.max_context, cfg.head_dim)
+        return torch.zeros(shape, dtype=self.embed.dtype, device=self.embed.device)
+
+    @torch.no_grad()
+    def forward(self, tokens, pos, cache):
+        """tokens int64 [M], pos int64 [M] (their positions) -> logits [M, vocab] (fp32)."""
+        h = self.embed.index_select(0, tokens)
+        cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
+        mask = self.arange[None, :] <= pos[:, None]
+        for i, block in enumerate(self.blocks):
+            h = block(h, cos, sin, pos, cache[i, 0], cache[i, 1], mask)
+        h = torch.nn.functional.rms_norm(h, (self.cfg.hidden,), self.final_norm, self.cfg.rms_eps)
+        return torch.nn.functional.linear(h[-1:], self.head).float()
+
+
+def random_mixnmatch_decoder(cfg: DecoderConfig, max_context: int, bit_choices: Sequence[int] = (2, 3, 4, 6, 8),
+                             seed: int = 0, dtype=torch.float16, device="cuda", zero_points: bool = True,
+                             keep_master: bool = False):
+    """A decoder with random master codes; every linear gets a bitwidth drawn from `bit_choices`
+    (seeded).  Returns `(decoder, layer_bits, masters)`: `layer_bits` maps `blocks.<i>.<name>` to
+    its bitwidth and `masters` (only with `keep_master`) to `(codes uint8 [N,K], scale, zero)`.
+    """
+    from matgptq_cuda.matgptq_linear import MatGPTQLinear
+
+    rnd = random.Random(seed)
+    gen = torch.Generator(device=device).manual_seed(seed)
+    layer_bits: Dict[str, int] = {}
+    masters = {}
+    blocks: List[Block] = []
+    for i in range(cfg.layers):
+        linears = {}
+        for name, (n, k) in cfg.linear_shapes().items():
+            bits = rnd.choice(list(bit_choices))
+            codes = torch.randint(0, 256, (n, k), dtype=torch.uint8, device=device, generator=gen)
+            groups = k // cfg.group_size
+            # scale chosen so that a linear roughly preserves the norm of its input
+            scale = ((torch.rand(n, groups, device=device, generator=gen) + 0.5) / (74.0 * k ** 0.5)).to(dtype)
+            zero = torch.randint(112, 144, (n, groups), device=device, generator=gen).to(dtype) if zero_points else None
+            linears[name] = MatGPTQLinear(matryoshka_slice(codes, 8, bits), scale, bits, cfg.group_size, zeros=zero)
+            layer_bits[f"blocks.{i}.{name}"] = bits
+            if keep_master:
+                masters[f"blocks.{i}.{name}"] = (codes, scale, zero)
+        blocks.append(Block(cfg, linears, dtype, device))
+    embed = (torch.randn(cfg.vocab, cfg.hidden, device=device, generator=gen)).to(dtype)
+    head = (torch.randn(cfg.vocab, cfg.hidden, device=device, generator=gen) * cfg.hidden ** -0.5).to(dtype)
+    return Decoder(cfg, blocks, embed, head, max_context), layer_bits, masters
+
+
+class DecodeSession:
+    """Greedy decoding with a static cache.  `prefill` runs the prompt in one pass (the M>16
+    kernels), `step` decodes one token eagerly, `capture` records `step` into a graph whose
+    replays read and advance device-side token and position tensors."""
+
+    def __init__(self, decoder: Decoder):
+        self.decoder = decoder
+        dev = decoder.embed.device
+        self.cache = decoder.new_cache()
+        self.token = torch.zeros(1, dtype=torch.int64, device=dev)
+        self.pos = torch.zeros(1, dtype=torch.int64, device=dev)
+        self.logits = torch.zeros(1, decoder.cfg.vocab, dtype=torch.float32, device=dev)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.stream = torch.cuda.Stream(device=dev)
+
+    def prefill(self, prompt: torch.Tensor) -> None:
+        n = prompt.numel()
+        if n + 1 > self.decoder.max_context:
+            raise ValueError("prompt longer than the cache")
+        pos = torch.arange(n, device=prompt.device)
+        logits = self.decoder(prompt.to(torch.int64), pos, self.cache)
+        self.logits.copy_(logits)
+        self.token.copy_(logits.argmax(dim=-1))
+        self.pos.fill_(n)
+
+    def _step_body(self) -> None:
+        logits = self.decoder(self.token, self.pos, self.cache)
+        self.logits.copy_(logits)
+        self.token.copy_(logits.argmax(dim=-1))
+        self.pos.add_(1)
+
+    def step(self) -> None:
+        """One token, eagerly.  The caller keeps `pos` below the cache length."""
+        self._step_body()
+
+    def capture(self) -> None:
+        """Records one step.  Token, position and cache are restored afterwards, so the capture
+        (and its eager warm-up) does not advance the sequence."""
+        saved = (self.token.clone(), self.pos.clone(), self.logits.clone())
+        row = self.cache[:, :, :, int(self.pos.item())].clone()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(self.stream):
+            self._step_body()  # warm-up on the capture stream: library workspaces exist before capture
+            self.stream.synchronize()
+            self.token.copy_(saved[0]); self.pos.copy_(saved[1])
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=self.stream):
+                self._step_body()
+            self.stream.synchronize()
+        self.token.copy_(saved[0]); self.pos.copy_(saved[1]); self.logits.copy_(saved[2])
+        self.cache[:, :, :, int(saved[1].item())] = row
+        torch.cuda.synchronize()
+        self.graph = graph
+
+    def replay(self) -> None:
+        self.graph.replay()
+
+    def generate(self, prompt: torch.Tensor, new_tokens: int, use_graph: bool = True) -> torch.Tensor:
+        """Greedy continuation of `prompt`: returns the `new_tokens` generated ids."""
+        if prompt.numel() + new_tokens > self.decoder.max_context:
+            raise ValueError("prompt + new_tokens exceed the cache")
+        self.prefill(prompt)
+        if use_graph and self.graph is None:
+            self.capture()
+        out = [self.token.clone()]
+        for _ in range(new_tokens - 1):
+            self.replay() if use_graph else self.step()
+            out.append(self.token.clone())
+        torch.cuda.synchronize()
+        return torch.cat(out)
+
+    def tokens_per_s(self, steps: int, use_graph: bool, repeats: int = 3) -> float:
+        """Best of `repeats` timings of `steps` consecutive tokens from the current position,
+        which is restored after each timing: every repeat sees the same context and the
+        session is left where it was."""
+        if int(self.pos.item()) + steps > self.decoder.max_context:
+            raise ValueError("not enough cache left for the timed steps")
+        if use_graph and self.graph is None:
+            self.capture()
+        run = self.replay if use_graph else self.step
+        saved = (self.token.clone(), self.pos.clone())
+        best = float("inf")
+        for _ in range(repeats):
+            self.token.copy_(saved[0]); self.pos.copy_(saved[1])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                run()
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        self.token.copy_(saved[0]); self.pos.copy_(saved[1])
+        return steps / best
+
+
+def measure(layers: int = 32, context: int = 512, new_tokens: int = 64, bit_choices: Sequence[int] = (2, 3, 4, 6, 8),
+            seed: int = 0, dtype=torch.float16) -> dict:
+    """Builds the random-weight decoder, prefills `context` tokens, and times decoding."""
+    cfg = DecoderConfig(layers=layers)
+    decoder, layer_bits, _ = random_mixnmatch_decoder(cfg, context + new_tokens + 8, bit_choices, seed, dtype)
+    session = DecodeSession(decoder)
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    prompt = torch.randint(0, cfg.vocab, (context,), device="cuda", generator=gen)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    session.prefill(prompt)
+    torch.cuda.synchronize()
+    first = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    session.prefill(prompt)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    eager = session.tokens_per_s(new_tokens, use_graph=False)
+    graph = session.tokens_per_s(new_tokens, use_graph=True)
+    shapes = cfg.linear_shapes()
+    weight_bytes = sum(shapes[name.rsplit(".", 1)[1]][0] * shapes[name.rsplit(".", 1)[1]][1] * b // 8
+                       for name, b in layer_bits.items())
+    hist: Dict[str, int] = {}
+    for b in layer_bits.values():
+        hist[str(b)] = hist.get(str(b), 0) + 1
+    return {"layers": layers, "context": context, "new_tokens": new_tokens, "dtype": str(dtype).replace("torch.", ""),
+            "bitwidth_histogram": dict(sorted(hist.items())),
+            "mean_bits": round(weight_bytes * 8 / sum(shapes[n.rsplit(".", 1)[1]][0] * shapes[n.rsplit(".", 1)[1]][1]
+                                                      for n in layer_bits), 2),
+            "prefill_ms": round(prefill_s * 1e3, 2), "first_prefill_ms": round(first * 1e3, 2),
+            "tokens_per_s_eager": round(eager, 1), "tokens_per_s_graph": round(graph, 1),
+            "ms_per_token_graph": round(1e3 / graph, 3),
+            "sliced_weight_GBps_graph": round(weight_bytes * graph / 1e9, 1)}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser(description="tokens/s of a random-weight Llama-3-8B-shaped Mix'n'Match decoder")
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--context", type=int, default=512)
+    ap.add_argument("--new_tokens", type=int, default=64)
+    ap.add_argument("--bits", type=int, nargs="+", default=[2, 3, 4, 6, 8])
+    ap.add_argument("--bf16", action="store_true")
+    args = ap.parse_args()
+    print(json.dumps(measure(args.layers, args.context, args.new_tokens, args.bits,
+                             dtype=torch.bfloat16 if args.bf16 else torch.float16)))
+
+
+if __name__ == "__main__":
+    main()
