@@ -167,16 +167,54 @@ class Decoder(torch.nn.Module):
         return torch.nn.functional.linear(h[-1:], self.head).float()
 
 
+class PluginLinear(torch.nn.Module):
+    """A linear driven the way vLLM drives a quantisation method (inference_lib/vllm_matgptq.py:
+    89-201): `create_weights`, the loader's copies into `qweight` / `scales`, then
+    `process_weights_after_loading`; `forward` is `apply`."""
+
+    def __init__(self, quant_config, prefix: str, codes: torch.Tensor, scale: torch.Tensor,
+                 zero: Optional[torch.Tensor]):
+        super().__init__()
+        import vllm_matgptq
+
+        n, k = codes.shape
+        self.layer = torch.nn.Module()
+        self.method = vllm_matgptq.MatGPTQLinearMethod(quant_config, quant_config.bitwidth_for(prefix))
+        self.method.create_weights(self.layer, k, [n], k, n, scale.dtype)
+        self.layer.to(codes.device)
+        self.layer.qweight.data.copy_(codes)
+        self.layer.scales.data.copy_(scale)
+        if zero is not None:
+            self.layer.zeros = torch.nn.Parameter(zero.clone(), requires_grad=False)
+        self.method.process_weights_after_loading(self.layer)
+        self.bitwidth = self.method.bitwidth
+
+    def forward(self, x):
+        return self.method.apply(self.layer, x)
+
+
 def random_mixnmatch_decoder(cfg: DecoderConfig, max_context: int, bit_choices: Sequence[int] = (2, 3, 4, 6, 8),
                              seed: int = 0, dtype=torch.float16, device="cuda", zero_points: bool = True,
-                             keep_master: bool = False):
+                             keep_master: bool = False, via_plugin: bool = False):
     """A decoder with random master codes; every linear gets a bitwidth drawn from `bit_choices`
     (seeded).  Returns `(decoder, layer_bits, masters)`: `layer_bits` maps `blocks.<i>.<name>` to
     its bitwidth and `masters` (only with `keep_master`) to `(codes uint8 [N,K], scale, zero)`.
+    With `via_plugin` the linears are built by the vLLM quantisation method, configured by a
+    `layer_bitwidths` map as a packed checkpoint would, instead of as `MatGPTQLinear` modules.
     """
     from matgptq_cuda.matgptq_linear import MatGPTQLinear
 
     rnd = random.Random(seed)
+    names = [f"blocks.{i}.{name}" for i in range(cfg.layers) for name in cfg.linear_shapes()]
+    drawn = {name: rnd.choice(list(bit_choices)) for name in names}
+    quant_config = None
+    if via_plugin:
+        import vllm_matgptq
+
+        quant_config = vllm_matgptq.MatGPTQConfig.from_config({
+            "group_size": cfg.group_size, "master_bitwidth": 8, "inference_bitwidth": 4,
+            "quant_dtype": str(dtype).replace("torch.", ""), "modules_to_not_convert": ["head"],
+            "layer_bitwidths": drawn})
     gen = torch.Generator(device=device).manual_seed(seed)
     layer_bits: Dict[str, int] = {}
     masters = {}
@@ -184,13 +222,17 @@ def random_mixnmatch_decoder(cfg: DecoderConfig, max_context: int, bit_choices: 
     for i in range(cfg.layers):
         linears = {}
         for name, (n, k) in cfg.linear_shapes().items():
-            bits = rnd.choice(list(bit_choices))
+            bits = drawn[f"blocks.{i}.{name}"]
             codes = torch.randint(0, 256, (n, k), dtype=torch.uint8, device=device, generator=gen)
             groups = k // cfg.group_size
             # scale chosen so that a linear roughly preserves the norm of its input
             scale = ((torch.rand(n, groups, device=device, generator=gen) + 0.5) / (74.0 * k ** 0.5)).to(dtype)
             zero = torch.randint(112, 144, (n, groups), device=device, generator=gen).to(dtype) if zero_points else None
-            linears[name] = MatGPTQLinear(matryoshka_slice(codes, 8, bits), scale, bits, cfg.group_size, zeros=zero)
+            if via_plugin:
+                linears[name] = PluginLinear(quant_config, f"blocks.{i}.{name}", codes, scale, zero)
+                assert linears[name].bitwidth == bits
+            else:
+                linears[name] = MatGPTQLinear(matryoshka_slice(codes, 8, bits), scale, bits, cfg.group_size, zeros=zero)
             layer_bits[f"blocks.{i}.{name}"] = bits
             if keep_master:
                 masters[f"blocks.{i}.{name}"] = (codes, scale, zero)
@@ -295,10 +337,11 @@ class DecodeSession:
 
 
 def measure(layers: int = 32, context: int = 512, new_tokens: int = 64, bit_choices: Sequence[int] = (2, 3, 4, 6, 8),
-            seed: int = 0, dtype=torch.float16) -> dict:
+            seed: int = 0, dtype=torch.float16, via_plugin: bool = True) -> dict:
     """Builds the random-weight decoder, prefills `context` tokens, and times decoding."""
     cfg = DecoderConfig(layers=layers)
-    decoder, layer_bits, _ = random_mixnmatch_decoder(cfg, context + new_tokens + 8, bit_choices, seed, dtype)
+    decoder, layer_bits, _ = random_mixnmatch_decoder(cfg, context + new_tokens + 8, bit_choices, seed, dtype,
+                                                      via_plugin=via_plugin)
     session = DecodeSession(decoder)
     gen = torch.Generator(device="cuda").manual_seed(seed)
     prompt = torch.randint(0, cfg.vocab, (context,), device="cuda", generator=gen)
@@ -320,6 +363,7 @@ def measure(layers: int = 32, context: int = 512, new_tokens: int = 64, bit_choi
     for b in layer_bits.values():
         hist[str(b)] = hist.get(str(b), 0) + 1
     return {"layers": layers, "context": context, "new_tokens": new_tokens, "dtype": str(dtype).replace("torch.", ""),
+            "linears": "vllm_matgptq.MatGPTQLinearMethod" if via_plugin else "MatGPTQLinear",
             "bitwidth_histogram": dict(sorted(hist.items())),
             "mean_bits": round(weight_bytes * 8 / sum(shapes[n.rsplit(".", 1)[1]][0] * shapes[n.rsplit(".", 1)[1]][1]
                                                       for n in layer_bits), 2),
@@ -336,9 +380,11 @@ def main() -> None:
     ap.add_argument("--new_tokens", type=int, default=64)
     ap.add_argument("--bits", type=int, nargs="+", default=[2, 3, 4, 6, 8])
     ap.add_argument("--bf16", action="store_true")
+    ap.add_argument("--modules", action="store_true", help="build the linears as MatGPTQLinear modules "
+                    "instead of through the vLLM quantisation method")
     args = ap.parse_args()
     print(json.dumps(measure(args.layers, args.context, args.new_tokens, args.bits,
-                             dtype=torch.bfloat16 if args.bf16 else torch.float16)))
+                             dtype=torch.bfloat16 if args.bf16 else torch.float16, via_plugin=not args.modules)))
 
 
 if __name__ == "__main__":

@@ -82,6 +82,22 @@ def test_graph_replays_equal_eager_steps():
     assert torch.equal(out, out_eager)
 
 
+def test_plugin_built_decoder_equals_module_built_decoder():
+    from matgptq_amd import decoder as D
+
+    cfg = D.DecoderConfig(**TINY)
+    a, bits_a, _ = D.random_mixnmatch_decoder(cfg, 64, seed=9)
+    b, bits_b, _ = D.random_mixnmatch_decoder(cfg, 64, seed=9, via_plugin=True)
+    assert bits_a == bits_b and len(set(bits_a.values())) >= 3
+    assert all(isinstance(blk.qkv, D.PluginLinear) for blk in b.blocks)
+    prompt = torch.randint(0, cfg.vocab, (20,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(4))
+    ta = D.DecodeSession(a).generate(prompt, 6, use_graph=True)
+    tb = D.DecodeSession(b).generate(prompt, 6, use_graph=True)
+    assert torch.equal(ta, tb)
+    pos = torch.arange(20, device="cuda")
+    assert torch.equal(a(prompt, pos, a.new_cache()), b(prompt, pos, b.new_cache()))
+
+
 def test_cache_limits_raise():
     D, cfg, dec, _, _ = _tiny(bit_choices=(4,), context=48)
     s = D.DecodeSession(dec)
