@@ -9,7 +9,7 @@ links the C ABI library `libmatgptq_hip.so`) and thereby registers
 
 with the schemas of the reference (inference_lib/matgptq_cuda/csrc/bindings.cpp:198-200)
 plus the additive ops documented in `matgptq_amd.ops`.  There is no fallback: when
-the libraries have not been built (`python -m matgptq_amd._build`), the import fails.
+the libraries have not been built (`python matgptq_amd/_build.py`), the import fails.
 """
 from __future__ import annotations
 
@@ -33,7 +33,7 @@ def load_extension():
         return sys.modules[name]
     if not os.path.exists(_EXT_PATH) or not os.path.exists(_lib.ABI_PATH):
         raise ImportError(
-            f"{_EXT_PATH} / {_lib.ABI_PATH} not built: run `python -m matgptq_amd._build` "
+            f"{_EXT_PATH} / {_lib.ABI_PATH} not built: run `python matgptq_amd/_build.py` "
             "(hipcc --offload-arch=gfx950); the HIP path has no fallback")
     import torch  # noqa: F401  (libtorch must be loaded before the extension)
 

@@ -36,7 +36,7 @@ def load() -> ctypes.CDLL:
         return _lib
     if not os.path.exists(ABI_PATH):
         raise MatGPTQError(
-            f"{ABI_PATH} is missing: build it with `python -m matgptq_amd._build` "
+            f"{ABI_PATH} is missing: build it with `python matgptq_amd/_build.py` "
             "(hipcc, --offload-arch=gfx950); there is no fallback path")
     L = ctypes.CDLL(ABI_PATH)
     vp, i64, ci, u32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint32

@@ -18,6 +18,8 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
   hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int S, int W, int kc,  \
                                 bool stream_flavour, size_t smem, hipStream_t);                \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);          \
+  hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, hipStream_t);   \
+  hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, hipStream_t); \
   hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
                                        int kc, bool stream_flavour, size_t smem, hipStream_t); \
   hipError_t launch_prefill_b##B##_bf16(const GemmArgs&, int group_size, int cfg, hipStream_t);
@@ -42,6 +44,8 @@ constexpr size_t kLdsBudget = 64 * 1024;  // dynamic LDS a decode workgroup may 
 
 struct Plan {
   bool decode;
+  bool skinny;   // mid-batch kernel (K split inside the workgroup), R row blocks per workgroup
+  int mb;        // mid-batch: blocks of 16 batch rows per workgroup
   int R, S, W;   // decode: row blocks per wave, slots and k-slices per workgroup
   int kc;        // decode: tiles of K staged in LDS at a time
   bool stream;   // decode: double-buffered flavour
@@ -62,7 +66,8 @@ size_t decode_lds_bytes(int R, int S, int W, int kc, int64_t M) {
 
 // Automatic choice; the flags word can override it for benchmarks:
 //   bits 8..15 : 0 = automatic, 1 + rsel + 3*shape = decode (rsel: R = 1,2,4; shape: kShapes),
-//                64 + cfg = prefill tile configuration
+//                64 + cfg = prefill tile configuration,
+//                80 + rsel + 3*(mb-1) = mid-batch kernel (rsel: R = 1,2,4; mb: 16 or 32 batch rows)
 //   bits 16..17: decode flavour, 0 = automatic, 1 = burst, 2 = stream
 int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp, uint32_t flags,
               Plan* p) {
@@ -70,6 +75,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   const int variant = (int)((flags & MATGPTQ_FLAG_VARIANT_MASK) >> MATGPTQ_FLAG_VARIANT_SHIFT);
   const int flavour = (int)((flags >> 16) & 3u);
   p->decode = M <= kDecodeMaxM;
+  p->skinny = false;
+  p->mb = 2;
   p->cfg = 0;
   // default decode shape (measured on MI355X, M = 1, Llama-3-8B layers): eight waves per
   // workgroup, all of them splitting K; four row blocks per wave once there are enough
@@ -91,19 +98,57 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
     // (bf16 storage has no ring loop: its 128 x 256 tile runs one wave per SIMD)
     if (wgs_big >= 448 && !(flags & MATGPTQ_FLAG_BF16)) p->cfg = 0;
-    else if (M <= 256) p->cfg = 4;
+    else if (M <= 512) p->cfg = 4;
     else p->cfg = 3;
+    // Mid-batch kernel (K split inside the workgroup) against the 32 x 128 tile, as measured on
+    // MI355X (4 bits, Llama-3-8B layers): the former dequantises every code once per 32 batch
+    // rows, about 2 us + 0.13 us per million codes and batch tile; the latter walks K serially,
+    // about 0.82 us per K tile while its workgroups fit the 512 resident slots and
+    // proportionally more beyond.
+    if (p->cfg == 4) {
+      const int64_t m_tiles = (M + 31) / 32;
+      const double mid = 2.0 + 0.13e-6 * (double)m_tiles * (double)N * (double)K;
+      const int64_t wgs = ((N + 127) / 128) * m_tiles;
+      const double walk = 0.82 * k_tiles * (wgs > 512 ? (double)wgs / 512.0 : 1.0);
+      p->skinny = mid < walk;
+    }
+  } else if (flavour == 0 && row_blocks < 1024 &&
+             (M >= 8 || (M >= 4 && k_tiles >= 64) || (M >= 2 && k_tiles >= 112))) {
+    // Small batches of layers with few rows: every decode workgroup stages the whole batch of
+    // activations (scaled copies, written by the vector ALU), which grows with M and K, while
+    // the mid-batch kernel copies them into LDS asynchronously.  Measured on MI355X (Llama-3-8B
+    // and 70B layers, 3 and 4 bits): the latter wins from these batch sizes on; on the layers
+    // with many rows the decode kernel stays ahead up to M = 16.
+    p->decode = false;
+    p->skinny = true;
+    p->mb = 1;
+  }
+  if (p->skinny) {
+    // as many row blocks per workgroup as still leave about 160 workgroups (the activations
+    // are re-read once per workgroup column)
+    const int64_t m_tiles = (M + 16 * p->mb - 1) / (16 * p->mb);
+    R = 1;
+    for (int r = 4; r > 1; r >>= 1)
+      if ((int64_t)((row_blocks + r - 1) / r) * m_tiles >= 160) { R = r; break; }
   }
   if (variant != 0) {
-    if (variant >= 64) {
+    if (variant >= 80) {
+      if (variant - 80 > 5) return MATGPTQ_EVARIANT;
+      p->decode = false;
+      p->skinny = true;
+      R = 1 << ((variant - 80) % 3);
+      p->mb = 1 + (variant - 80) / 3;
+    } else if (variant >= 64) {
       if (variant - 64 > 7) return MATGPTQ_EVARIANT;
       p->decode = false;
+      p->skinny = false;
       p->cfg = variant - 64;
     } else {
       if (M > kDecodeMaxM) return MATGPTQ_EVARIANT;
       const int v = variant - 1;
       if (v >= 3 * kNumShapes) return MATGPTQ_EVARIANT;
       p->decode = true;
+      p->skinny = false;
       R = 1 << (v % 3);
       S = kShapes[v / 3][0];
       W = kShapes[v / 3][1];
@@ -114,6 +159,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     // the prefill kernel addresses X through a 32-bit buffer offset
     if ((uint64_t)M * (uint64_t)K * 2u >= (1ull << 32)) return MATGPTQ_ESIZE;
     p->R = p->S = p->W = p->kc = 0;
+    // (four row blocks per workgroup only up to 6 bits and one scale per tile: register budget)
+    if (p->skinny) p->R = R >= 4 && (group_size == 32 || bits > 6) ? 2 : R;
     p->stream = false;
     p->smem = 0;
     return MATGPTQ_OK;
@@ -173,6 +220,19 @@ hipError_t launch_prefill(int bits, bool bf16, const GemmArgs& a, int g, const P
 #undef MATGPTQ_CASE
 }
 
+hipError_t launch_skinny(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+#define MATGPTQ_CASE(B) \
+  case B: return bf16 ? launch_skinny_b##B##_bf16(a, g, p.R, p.mb, s) : launch_skinny_b##B(a, g, p.R, p.mb, s);
+  switch (bits) {
+    MATGPTQ_CASE(2)
+    MATGPTQ_CASE(3)
+    MATGPTQ_CASE(4)
+    MATGPTQ_CASE(6)
+    default: return bf16 ? launch_skinny_b8_bf16(a, g, p.R, p.mb, s) : launch_skinny_b8(a, g, p.R, p.mb, s);
+  }
+#undef MATGPTQ_CASE
+}
+
 }  // namespace
 }  // namespace matgptq
 
@@ -221,8 +281,9 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
   a.row_blocks = (int)(N / 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
-  const hipError_t err = p.decode ? launch_decode(bitwidth, bf16, a, group_size, p, s)
-                                  : launch_prefill(bitwidth, bf16, a, group_size, p, s);
+  const hipError_t err = p.decode   ? launch_decode(bitwidth, bf16, a, group_size, p, s)
+                         : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, s)
+                                    : launch_prefill(bitwidth, bf16, a, group_size, p, s);
   if (err != hipSuccess) return MATGPTQ_ELAUNCH;
   if (!(flags & MATGPTQ_FLAG_ASYNC)) {
     if (hipStreamSynchronize(s) != hipSuccess) return MATGPTQ_ELAUNCH;
@@ -241,6 +302,9 @@ int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, in
     snprintf(buf, buf_len, "decode-%s b%d g%d zp%d R%d S%d W%d kc%d lds%zu",
              p.kc < (int)(K / 128) ? "chunked" : (p.stream ? "stream" : "burst"), bitwidth, group_size,
              has_zeros ? 1 : 0, p.R, p.S, p.W, p.kc, p.smem);
+  else if (p.skinny)
+    snprintf(buf, buf_len, "midbatch b%d g%d zp%d R%d mb%d", bitwidth, group_size, has_zeros ? 1 : 0,
+             p.R, p.mb);
   else
     snprintf(buf, buf_len, "prefill b%d g%d zp%d cfg%d", bitwidth, group_size, has_zeros ? 1 : 0,
              p.cfg);

@@ -49,43 +49,6 @@ constexpr int kXs = 64;          // activation columns per LDS stage
 #endif
 constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 
-// One raw pair -> two weights.  u = c - 2^(b-1) is exact.
-//   symmetric, fp16 storage:  w = u * (scale * m),  m = 2^(8-b) (a power of two: one rounding,
-//     the value the reference's dequantize() gives);
-//   zero point, fp16 storage: w = fma(u, scale * m, -(scale * zrel)),  zrel = zero - 128: two
-//     instructions per pair instead of three.  scale * zrel is rounded to fp16 before the fma,
-//     so w can differ from dequantize()'s  fp16(scale * fp16(m u - zrel))  by one rounding of a
-//     term no larger than 128 scale: at most scale / 16, less than the rounding error of w
-//     itself (the dense dequantize_matgptq operator keeps the reference's exact sequence);
-//   bf16 storage: a bf16 scale can lie far below fp16's normal range, so the caller passes
-//     scale * 2^8 and zrel * 2^-8 and  v = m u 2^-8 - zrel 2^-8  is formed exactly and
-//     multiplied by the scale (the symmetric form takes the same route with zrel = 0).
-// `a`, `b`: (scale * m, scale * zrel) for fp16 storage with zero points, (scale', zrel') else.
-template <int BITS, int P, bool ZP>
-__device__ __forceinline__ half2v dequant_pair(uint32_t raw, half2v b, half2v a) {
-  const half2v u = centre_raw<P>(raw, Codec<BITS>::kCentre);
-  if constexpr (kBf16) {
-    constexpr float m = (float)(1 << (8 - BITS)) / 256.0f;
-    const half2v v = __builtin_elementwise_fma(u, h2_splat(m), -b);
-    return v * a;
-  } else if constexpr (ZP) {
-    return __builtin_elementwise_fma(u, a, -b);
-  } else {
-    return u * a;
-  }
-}
-
-template <int BITS, int J, bool ZP>
-__device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const UnpackConsts<BITS>& k,
-                                              half2v zrel, half2v scale, Frag& a) {
-  uint32_t raw[4];
-  raw_octet<BITS, J>(w, k, raw);
-  a.p[0] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 0), ZP>(raw[0], zrel, scale);
-  a.p[1] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 1), ZP>(raw[1], zrel, scale);
-  a.p[2] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 2), ZP>(raw[2], zrel, scale);
-  a.p[3] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 3), ZP>(raw[3], zrel, scale);
-}
-
 // Two waves per SIMD (256 registers each) whenever the accumulators leave room for the rest:
 // one wave alone cannot keep the matrix pipe busy.  The tile whose accumulators take half of
 // that budget runs the ring loop below (activations straight into LDS, one operand set).

@@ -1,0 +1,297 @@
+// Mid-batch kernel (16 < M <= a few hundred): the K dimension is split inside the workgroup.
+// Compiled once per bitwidth with -DMATGPTQ_BITS=b.
+//
+// At these batch sizes a layer has few output tiles: a kernel that gives every workgroup a
+// tile of outputs and walks K serially leaves most of the GPU idle and is bound by the latency
+// of one K walk (the reference's tensor-core kernel has this shape, one 16 x 8 tile per block,
+// inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:337-634).  Here
+//
+//  * a workgroup of eight waves owns R row blocks of 16 weight rows and 16*MB activation rows;
+//    wave w takes the K tiles w, w + 8, ... of those rows, so a layer with N / (16 R) x M / (16 MB)
+//    output tiles still runs eight times as many waves, each with a short K walk;
+//  * each wave dequantises its tiles from registers into the 16x32 MFMA operand (the same
+//    arithmetic as the large-batch kernel).  No two waves of a workgroup read the same
+//    activations, so every wave stages its own: buffer_load ... lds copies the 16*MB x 128
+//    activations of a tile from global memory straight into one of the wave's private LDS
+//    buffers, 256 contiguous bytes per 16 lanes (an operand read straight from global memory
+//    would touch sixteen rows with sixteen adjacent lanes).  16-byte chunk c of row r lies at
+//    position c ^ (r & 15) of the LDS row, so the sixteen lanes of an operand read hit sixteen
+//    different bank groups;
+//  * a wave keeps a ring of 4 / MB stages (an LDS buffer and a register set of codes, scales
+//    and zeros each) and requests a tile as many tiles ahead: a walk is short (K / 1024
+//    tiles), so what hides the memory latency is the depth of that ring, not a long loop.
+//    Only the wave itself waits for its copies (vmcnt, counted by hand: every stage issues the
+//    same number of instructions, so "all but the youngest stages" is a constant); there is no
+//    barrier in the loop;
+//  * every load is branch-free (tiles beyond K, rows beyond M or N go through a zero-length
+//    buffer descriptor or an out-of-range offset);
+//  * the eight partial sums meet in LDS once, at the end; the threads add them and store four
+//    consecutive output columns each.
+//
+// The activations are re-read once per workgroup column (N / (16 R) times in total, from L2):
+// that traffic, not the weights, bounds this kernel, which is why R grows with N.
+#include "device_common.h"
+
+#ifndef MATGPTQ_BITS
+#error "compile with -DMATGPTQ_BITS={2,3,4,6,8}"
+#endif
+
+namespace matgptq {
+
+namespace {
+
+constexpr int kBits = MATGPTQ_BITS;
+constexpr int kWaves = 8;
+
+// Stages of a wave's ring: as many as fit 128 KB of LDS per workgroup.
+constexpr int skinny_stages(int mb) { return 4 / mb; }
+
+// LDS of a workgroup: per wave and stage an activation buffer of 16*MB rows x 256 bytes; the
+// partial sums (16 bytes per lane, row block and batch block per wave) reuse them after the loop.
+constexpr int skinny_lds_bytes(int r, int mb) {
+  const int stage = kWaves * skinny_stages(mb) * mb * 16 * 256, sums = kWaves * r * mb * 64 * 16;
+  return stage > sums ? stage : sums;
+}
+
+template <int BITS, int GROUP, bool ZP, int R, int MB>
+__global__ void __launch_bounds__(64 * kWaves, 2)
+skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
+  constexpr int GPT = GROUP == 32 ? 4 : 1;
+  constexpr int kStage = MB * 16 * 256;  // bytes of one activation buffer
+  constexpr int NS = skinny_stages(MB);  // stages of the ring; a tile is requested NS - 1 tiles ahead
+  // vector-memory instructions of one stage: activation copies, then codes, scales, zeros
+  constexpr int kIssue = 4 * MB + R * (tile_load_count(BITS) + GPT * (ZP ? 2 : 1));
+  __shared__ __align__(16) unsigned char smem[skinny_lds_bytes(R, MB)];  // (this target has 160 KB per workgroup)
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15;
+  const int q = lane >> 4;
+
+  // Workgroup ids go round-robin over the 8 XCDs: remapped so that the workgroups of one XCD
+  // walk consecutive activation tiles of the same weight rows and share those rows in its L2.
+  const int total = n_tiles * m_tiles;
+  int lid = blockIdx.x;
+  if ((total & 7) == 0) lid = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+  const int nt = lid / m_tiles;
+  const int m0 = (lid - nt * m_tiles) * (16 * MB);
+  const int rb_first = nt * R;
+
+  constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
+  const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
+  const uint32_t w_bytes = (uint32_t)a.row_blocks * rb_bytes;
+  const uint32_t aux_bytes = (uint32_t)a.row_blocks * a.G * 32;  // scales / zeros: [N/16][G][16] halves
+  const uint32_t x_bytes = (uint32_t)a.M * (uint32_t)a.K * 2u;
+
+  float4v acc[R][MB];
+#pragma unroll
+  for (int rr = 0; rr < R; rr++)
+#pragma unroll
+    for (int i = 0; i < MB; i++) acc[rr][i] = float4v{0.f, 0.f, 0.f, 0.f};
+
+  const UnpackConsts<BITS> kc_unpack;
+  // codes, scales and zeros of every stage; scales and zeros stay as loaded and are converted
+  // where they are used
+  uint32_t wr[NS][R][BITS], sr[NS][R][GPT], zr[NS][R][GPT];
+
+  auto load_weights = [&](uint32_t (&w)[R][BITS], uint32_t (&s)[R][GPT], uint32_t (&z)[R][GPT], int kb) {
+#pragma unroll
+    for (int rr = 0; rr < R; rr++) {
+      const int rb = rb_first + rr;
+      const bool valid = rb < a.row_blocks && kb < a.k_tiles;
+      const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
+      const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
+      const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
+      load_tile_words<BITS, 0>(wr, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
+#pragma unroll
+      for (int gg = 0; gg < GPT; gg++) {
+        const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
+        const uint32_t so = ((uint32_t)rb * a.G + g) * 32;  // bytes
+        s[rr][gg] = __builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0);
+        if constexpr (ZP) z[rr][gg] = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
+        else z[rr][gg] = 0u;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // Copy of one tile's activations: instruction i moves rows 4i .. 4i+3 (lane l: row 4i + l/16,
+  // LDS position l%16, which holds chunk (l%16) ^ (row & 15) of the row's 256 bytes).
+  unsigned char* const stage = smem + wave * (NS * kStage);
+  uint32_t dma_voff[4 * MB];
+#pragma unroll
+  for (int i = 0; i < 4 * MB; i++) {
+    const int row = 4 * i + (lane >> 4);
+    const int c = (lane & 15) ^ (row & 15);
+    const uint32_t m = (uint32_t)(m0 + row);
+    dma_voff[i] = m < (uint32_t)a.M ? m * (uint32_t)a.K * 2u + c * 16 : x_bytes;
+  }
+  auto dma = [&](int buf, int kb) {
+    const BufRsrc xres = make_rsrc(a.x, kb < a.k_tiles ? x_bytes : 0u);
+#pragma unroll
+    for (int i = 0; i < 4 * MB; i++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          xres, (__attribute__((address_space(3))) void*)(stage + buf * kStage + i * 1024), 16, (int)dma_voff[i],
+          (int)((uint32_t)kb * 256u), 0, 0);  // (int: the builtin's own parameter type)
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // operand of batch rows i*16 + r16, columns [j*32 + q*8, +8) of the tile: chunk 4j + q
+  auto read_frag = [&](int buf, int i, int j) {
+    const half8 raw = *reinterpret_cast<const half8*>(stage + buf * kStage + (i * 16 + r16) * 256 +
+                                                      (((4 * j + q) ^ r16) * 16));
+    return storage8_to_half8(raw);
+  };
+
+  auto dequant_step = [&](Frag (&aw)[R], const uint32_t (&w)[R][BITS], const uint32_t (&s)[R][GPT],
+                          const uint32_t (&z)[R][GPT], auto jtag) {
+    constexpr int J = decltype(jtag)::value;
+#pragma unroll
+    for (int rr = 0; rr < R; rr++) {
+      const int gg = GROUP == 32 ? J : 0;
+      // fp16 storage: scale * 2^(8-b) and scale * (zero - 128);
+      // bf16 storage: scale * 2^8 and (zero - 128) * 2^-8, converted through fp32
+      _Float16 s1, z1 = (_Float16)0.f;
+      if constexpr (kBf16) {
+        s1 = (_Float16)(bf16_bits_to_float(s[rr][gg]) * 256.0f);
+        if constexpr (ZP) z1 = (_Float16)((bf16_bits_to_float(z[rr][gg]) - 128.0f) * (1.0f / 256.0f));
+      } else {
+        const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)s[rr][gg]);
+        s1 = (_Float16)((float)s0 * (float)(1 << (8 - BITS)));  // scale * m
+        if constexpr (ZP) z1 = s0 * (__builtin_bit_cast(_Float16, (uint16_t)z[rr][gg]) - (_Float16)128.0f);
+      }
+      const half2v sc = {s1, s1};
+      const half2v zr = {z1, z1};
+      dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
+    }
+  };
+
+  // Tile t of the walk (K tile kb = wave + 8 t) lives in stage t % NS (`btag`).  Stages are
+  // issued in tile order, NS - 1 tiles ahead, kIssue instructions each: at the start of tile t
+  // everything up to stage t must have arrived and the NS - 2 younger stages may be in flight.
+  auto issue = [&](auto btag, int kb) {
+    constexpr int B = decltype(btag)::value;
+    dma(B, kb);
+    load_weights(wr[B], sr[B], zr[B], kb);
+  };
+  auto tile = [&](int t, auto btag) {
+    constexpr int B = decltype(btag)::value;
+    const int kb = wave + t * kWaves;
+    // (the counter holds 63 at most: waiting for fewer in flight than necessary is safe)
+    constexpr int n = (NS - 2) * kIssue < 63 ? (NS - 2) * kIssue : 63;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt((n & 15) | (7 << 4) | (0 << 8) | ((n >> 4) << 14));  // vmcnt(n), lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    // the stage of tile t - 1 is free: its operands have been read, its codes dequantised
+    issue(std::integral_constant<int, (B + NS - 1) % NS>{}, kb + (NS - 1) * kWaves);
+    if (kb < a.k_tiles) {
+      auto one = [&](auto jtag) {
+        constexpr int J = decltype(jtag)::value;
+        Frag aw[R];
+        dequant_step(aw, wr[B], sr[B], zr[B], jtag);
+#pragma unroll
+        for (int i = 0; i < MB; i++) {
+          const half8 b = read_frag(B, i, J);
+#pragma unroll
+          for (int rr = 0; rr < R; rr++)
+            acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b, acc[rr][i], 0, 0, 0);
+        }
+      };
+      one(std::integral_constant<int, 0>{});
+      one(std::integral_constant<int, 1>{});
+      one(std::integral_constant<int, 2>{});
+      one(std::integral_constant<int, 3>{});
+    }
+    // (the next tile's wait must not move above this tile's operand reads)
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const int walk = (a.k_tiles + kWaves - 1) / kWaves;  // tiles of the longest walk
+  __builtin_amdgcn_sched_barrier(0);
+  issue(std::integral_constant<int, 0>{}, wave);
+  if constexpr (NS == 4) {
+    issue(std::integral_constant<int, 1>{}, wave + kWaves);
+    issue(std::integral_constant<int, 2>{}, wave + 2 * kWaves);
+  }
+  for (int t = 0; t < walk; t += NS) {
+    tile(t, std::integral_constant<int, 0>{});
+    tile(t + 1, std::integral_constant<int, 1>{});
+    if constexpr (NS == 4) {
+      tile(t + 2, std::integral_constant<int, 2>{});
+      tile(t + 3, std::integral_constant<int, 3>{});
+    }
+  }
+
+  // The eight partial sums of every output meet in LDS (over the activation buffers: every
+  // wave has to be done with its own first); thread t adds the eight float4 of one (row
+  // block, batch block, lane) and stores rows (weight rows) 4q..4q+3 of column (batch row) r16.
+  __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));  // nothing in flight into LDS any more
+  __syncthreads();
+  float4v* const red = reinterpret_cast<float4v*>(smem);
+#pragma unroll
+  for (int rr = 0; rr < R; rr++)
+#pragma unroll
+    for (int i = 0; i < MB; i++) red[((wave * R + rr) * MB + i) * 64 + lane] = acc[rr][i];
+  __syncthreads();
+  if (tid < R * MB * 64) {
+    float4v sum = red[tid];
+#pragma unroll
+    for (int w = 1; w < kWaves; w++) sum += red[w * R * MB * 64 + tid];
+    const int l = tid & 63, ri = tid >> 6;
+    const int rb = rb_first + ri / MB;
+    const int m = m0 + (ri % MB) * 16 + (l & 15);
+    if (rb < a.row_blocks && m < a.M) {
+      uint16_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) o[e] = float_to_storage(sum[e]);
+      *reinterpret_cast<uint2*>(a.y + (size_t)m * a.N + (size_t)rb * 16 + 4 * (l >> 4)) =
+          make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+    }
+  }
+}
+
+template <int GROUP, bool ZP, int R, int MB>
+hipError_t launch_r(const GemmArgs& a, hipStream_t stream) {
+  const int n_tiles = (a.row_blocks + R - 1) / R;
+  const int m_tiles = (a.M + 16 * MB - 1) / (16 * MB);
+  const dim3 grid(n_tiles * m_tiles), block(64 * kWaves);
+  hipLaunchKernelGGL((skinny_kernel<kBits, GROUP, ZP, R, MB>), grid, block, 0, stream, a, n_tiles, m_tiles);
+  return hipGetLastError();
+}
+
+template <int GROUP, bool ZP, int MB>
+hipError_t launch_rows(const GemmArgs& a, int r, hipStream_t s) {
+  // (four row blocks fit the register budget of two waves per SIMD up to 6 bits and with one
+  // scale and zero per tile and row block; group 32 carries four)
+  if constexpr (GROUP != 32 && kBits <= 6) {
+    if (r >= 4) return launch_r<GROUP, ZP, 4, MB>(a, s);
+  }
+  if (r >= 2) return launch_r<GROUP, ZP, 2, MB>(a, s);
+  return launch_r<GROUP, ZP, 1, MB>(a, s);
+}
+
+template <int GROUP, bool ZP>
+hipError_t launch_batch(const GemmArgs& a, int r, int mb, hipStream_t s) {
+  return mb >= 2 ? launch_rows<GROUP, ZP, 2>(a, r, s) : launch_rows<GROUP, ZP, 1>(a, r, s);
+}
+
+}  // namespace
+
+#define MATGPTQ_CAT2(a, b) a##b
+#define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
+// r: row blocks of 16 weight rows per workgroup (1, 2 or 4); mb: blocks of 16 batch rows (1 or 2)
+#if MATGPTQ_BF16
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(MATGPTQ_CAT(launch_skinny_b, MATGPTQ_BITS), _bf16)
+#else
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_skinny_b, MATGPTQ_BITS)
+#endif
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int r, int mb, hipStream_t stream) {
+  const bool zp = a.zeros != nullptr;
+  if (group_size == 128)
+    return zp ? launch_batch<128, true>(a, r, mb, stream) : launch_batch<128, false>(a, r, mb, stream);
+  if (group_size == 32)
+    return zp ? launch_batch<32, true>(a, r, mb, stream) : launch_batch<32, false>(a, r, mb, stream);
+  return zp ? launch_batch<-1, true>(a, r, mb, stream) : launch_batch<-1, false>(a, r, mb, stream);
+}
+
+}  // namespace matgptq

@@ -14,6 +14,7 @@ from tests import _gpu_util as G
 pytestmark = pytest.mark.gpu
 BITS = (2, 3, 4, 6, 8)
 GROUPS = (128, 32, -1)
+DECODE_KERNEL = 1 | (1 << 8)  # flags: asynchronous, decode kernel forced (one row block per wave, eight K slices)
 
 
 @pytest.mark.parametrize("b", BITS)
@@ -85,10 +86,13 @@ def test_forward_against_reference_vectors(b, golden):
 @pytest.mark.parametrize("g", GROUPS)
 @pytest.mark.parametrize("b", BITS)
 def test_decode_parity(b, g, zp):
+    # the default choice (from some batch size on the mid-batch kernel) and the decode kernel forced
     lay = G.Layer(64, 1024, b, g, seed=b, zero_points=zp)
     for m in (1, 2, 3, 5, 8, 16):
         x = o.make_activations(m, 1024, seed=m)
-        G.assert_close_to_oracle(lay.run(x), x, lay.w, f"decode b={b} g={g} zp={zp} M={m}")
+        G.assert_close_to_oracle(lay.run(x), x, lay.w, f"small batch b={b} g={g} zp={zp} M={m}")
+        G.assert_close_to_oracle(lay.run(x, flags=DECODE_KERNEL), x, lay.w, f"decode b={b} g={g} zp={zp} M={m}")
+    assert _lib.describe_plan(b, g, 64, 1024, 16, zp, DECODE_KERNEL).startswith("decode")
 
 
 @pytest.mark.parametrize("zp", (False, True))
@@ -128,6 +132,54 @@ def test_prefill_ring_tile_every_format(b, g, zp):
     assert _lib.describe_plan(b, g, n, k, m, zp, 1 | (64 << 8)).endswith("cfg0")
 
 
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_midbatch_kernel_every_format(b, g, zp):
+    # K split over the eight waves of a workgroup: 13 K tiles (ragged split, odd walk), 19 row
+    # blocks (ragged for 2 and 4 row blocks per workgroup), ragged batch
+    n, k, m = 304, 128 * 13, 77
+    lay = G.Layer(n, k, b, g, seed=17 * b + (g & 7), zero_points=zp)
+    x = o.make_activations(m, k, seed=b + 1)
+    for rsel in range(6):
+        flags = 1 | ((80 + rsel) << 8)
+        y = lay.run(x, flags=flags)
+        G.assert_close_to_oracle(y, x, lay.w, f"mid-batch b={b} g={g} zp={zp} rsel={rsel}")
+        assert _lib.describe_plan(b, g, n, k, m, zp, flags).startswith("midbatch")
+
+
+@pytest.mark.parametrize("m", (17, 32, 33, 64, 128, 250))
+@pytest.mark.parametrize("n,k", [(4096, 4096), (512, 14336), (1040, 384)])
+def test_midbatch_kernel_shapes(n, k, m):
+    # long and short K walks (K = 384: five of the eight waves have no tile at all)
+    lay = G.Layer(n, k, 4, 128, seed=n + m)
+    x = o.make_activations(m, k, seed=m)
+    rows = np.r_[0:min(m, 24), max(m - 24, 0):m]
+    for rsel in range(6):
+        y = lay.run(x, flags=1 | ((80 + rsel) << 8))
+        G.assert_close_to_oracle(y[rows], x[rows], lay.w, f"mid-batch {n}x{k} M={m} rsel={rsel}")
+
+
+def test_midbatch_kernel_agrees_with_prefill_tile_closely():
+    # same products, different summation order (eight partial sums): outputs agree to fp32
+    # rounding of the accumulation, far inside one fp16 rounding of most outputs
+    n, k, m, b, g = 2048, 4096, 96, 4, 128
+    lay = G.Layer(n, k, b, g, seed=5)
+    x = o.make_activations(m, k, seed=6)
+    a = lay.run(x, flags=1 | (81 << 8)).astype(np.float64)
+    c = lay.run(x, flags=1 | (68 << 8)).astype(np.float64)
+    scale = np.max(np.abs(c))
+    assert np.max(np.abs(a - c)) <= 2.0 ** -9 * scale
+    assert np.mean(a == c) > 0.9
+
+
+def test_midbatch_kernel_outlier_channels():
+    lay = G.Layer(512, 4096, 3, 128, seed=12)
+    x = o.make_activations(48, 4096, seed=3, outlier_frac=0.01, outlier_gain=20.0)
+    for rsel in range(6):
+        G.assert_close_to_oracle(lay.run(x, flags=1 | ((80 + rsel) << 8)), x, lay.w, f"outliers rsel={rsel}")
+
+
 def test_decode_every_work_split():
     # all (R, S, W) shapes in both flavours; 65 row blocks leave idle slots in the last
     # workgroup, K = 4096 gives up to 32 tiles per wave
@@ -152,14 +204,16 @@ def test_small_batch_with_outlier_channels(b, m):
     lay = G.Layer(256, 4096, b, 128, seed=30 + m)
     x = o.make_activations(m, 4096, seed=m, outlier_frac=0.01, outlier_gain=20.0)
     G.assert_close_to_oracle(lay.run(x), x, lay.w, f"outliers b={b} M={m}")
+    G.assert_close_to_oracle(lay.run(x, flags=DECODE_KERNEL), x, lay.w, f"outliers, decode kernel b={b} M={m}")
 
 
 def test_chunked_activation_staging():
     # M = 16 with K = 14336 does not fit in LDS at once: the kernel walks K in chunks
     lay = G.Layer(64, 14336, 4, 128, seed=7)
     x = o.make_activations(16, 14336, seed=7)
-    assert _lib.describe_plan(4, 128, 64, 14336, 16, True).startswith("decode-chunked")
-    G.assert_close_to_oracle(lay.run(x), x, lay.w, "chunked")
+    assert _lib.describe_plan(4, 128, 64, 14336, 16, True, DECODE_KERNEL).startswith("decode-chunked")
+    G.assert_close_to_oracle(lay.run(x, flags=DECODE_KERNEL), x, lay.w, "chunked")
+    G.assert_close_to_oracle(lay.run(x), x, lay.w, "default choice")
 
 
 @pytest.mark.parametrize("gsz", (-1, 32, 128))
@@ -180,8 +234,9 @@ def test_reference_kernel_test_grid(b, k, m, gsz):
     expect = o.linear_f64(x, w).astype(np.float16)
     pk = G.pack_device(codes, b, from_master=False)
     sd = G.reorder_device(scales, n, k, gsz)
-    y = G.gemm(b, gsz, n, k, G.to_dev(x), pk, sd, None).cpu().numpy()
-    assert np.array_equal(y.view(np.uint16), expect.view(np.uint16))
+    for flags in (1, DECODE_KERNEL):
+        y = G.gemm(b, gsz, n, k, G.to_dev(x), pk, sd, None, flags=flags).cpu().numpy()
+        assert np.array_equal(y.view(np.uint16), expect.view(np.uint16)), flags
 
 
 LLAMA8B = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "down": (4096, 14336)}
@@ -317,8 +372,24 @@ def test_reference_kernel_test_grid_bf16(b, k, m, gsz):
     w = (codes.astype(np.float64) - (1 << (b - 1))) * np.repeat(scales, g, axis=1) * (1 << (8 - b))
     expect = o.round_to_bf16(o.linear_f64(x, w))
     pk = G.pack_device(codes, b, from_master=False)
-    y = _gemm_bf16(b, gsz, n, k, x, pk, scales, None)
-    assert np.array_equal(y.view(np.uint32), expect.view(np.uint32))
+    for flags in (3, DECODE_KERNEL | 2):
+        y = _gemm_bf16(b, gsz, n, k, x, pk, scales, None, flags=flags)
+        assert np.array_equal(y.view(np.uint32), expect.view(np.uint32)), flags
+
+
+@pytest.mark.parametrize("b,g,zp", [(4, 128, True), (3, 32, True), (8, 128, False), (2, -1, True), (6, 32, False)])
+def test_bf16_midbatch_kernel(b, g, zp):
+    n, k, m = 304, 128 * 13, 77
+    q, s16, z16 = o.make_layer(n, k, g, seed=70 + b, symmetric=not zp)
+    s = o.round_to_bf16(s16.astype(np.float32))
+    z = z16.astype(np.float32)
+    x = o.round_to_bf16(o.make_activations(m, k, seed=9).astype(np.float32))
+    pk = G.pack_device(q, b, True)
+    ref = o.linear_f64(x, o.dequantize_bf16(q, s, z, b, g))
+    for rsel in range(6):
+        y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | ((80 + rsel) << 8))
+        assert np.all(np.isfinite(y))
+        assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref)), (b, g, zp, rsel)
 
 
 @pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8)))
