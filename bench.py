@@ -218,20 +218,34 @@ def main() -> int:
                     }
                 del ring
         extra["gemv_M1"] = table
-        # ----------------------------------------------------------- small batch
+        # ----------------------------------------- small batch (configs[2]), all four layers
         small = {}
-        for m in (2, 4, 8, 16):
+        for name, (n, k) in LLAMA3_8B.items():
             for b in (4, 3):
-                name = "gate_up"
-                n, k = LLAMA3_8B[name]
                 ring = rings[name] if b == bits else make_ring(n, k, b, max(2, int(RING_BYTES // (n * k * b // 8)) + 1))
                 cp = len(ring)
+                for m in (2, 4, 8, 16):
+                    xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+                    ym = torch.empty(m, n, dtype=torch.float16, device=dev)
+                    t = timed_graph(lambda: [launch(b, n, k, xm, ring[i % cp], aux[name][0], aux[name][1], ym)
+                                             for i in range(cp)]) / cp
+                    small[f"{name}_b{b}_M{m}"] = {"us": round(t * 1e6, 2),
+                                                  "weight_GBps": round(n * k * b / 8 / t / 1e9, 1),
+                                                  "kernel": _lib.describe_plan(b, GROUP, n, k, m, True).split()[0]}
+                del ring
+        # -------------------------------------------- mid batch: between decode and prefill
+        mid = {}
+        for name, (n, k) in LLAMA3_8B.items():
+            ring = rings[name]
+            cp = len(ring)
+            for m in (32, 64, 128, 256):
                 xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
                 ym = torch.empty(m, n, dtype=torch.float16, device=dev)
-                t = timed_graph(lambda: [launch(b, n, k, xm, ring[i % cp], aux[name][0], aux[name][1], ym)
+                t = timed_graph(lambda: [launch(bits, n, k, xm, ring[i % cp], aux[name][0], aux[name][1], ym)
                                          for i in range(cp)]) / cp
-                small[f"gate_up_b{b}_M{m}"] = {"us": round(t * 1e6, 2),
-                                               "weight_GBps": round(n * k * b / 8 / t / 1e9, 1)}
+                mid[f"{name}_b4_M{m}"] = {"us": round(t * 1e6, 2), "TFLOPs": round(2.0 * m * n * k / t / 1e12, 1),
+                                          "kernel": _lib.describe_plan(bits, GROUP, n, k, m, True).split()[0]}
+        extra["mid_batch"] = mid
         extra["small_batch"] = small
         del rings
         torch.cuda.empty_cache()
