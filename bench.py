@@ -58,10 +58,11 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
-    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill"),
+    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill", "midbatch"),
                     help="for rocprofv3 --pmc runs.  decode: launch only the dominant kernel over the ring of "
                          "weight copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's "
-                         "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer")
+                         "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer.  "
+                         "midbatch: launch only the mid-batch kernel, 4096->4096 at M=64 and 14336->4096 at M=16")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -131,6 +132,22 @@ def main() -> int:
                 launch(bits, n, k, x, packed, sc, zr, y)
             stream.synchronize()
         print(json.dumps({"counter_pass": _lib.describe_plan(bits, GROUP, n, k, 2048, True), "launches": 6}))
+        return 0
+    if args.counter_pass == "midbatch":
+        plans = []
+        for name, m in (("o", 64), ("down", 16)):
+            n, k = LLAMA3_8B[name]
+            copies = 16
+            ring = make_ring(n, k, bits, copies)
+            sc, zr = make_aux(n, k)
+            x = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+            y = torch.empty(m, n, dtype=torch.float16, device=dev)
+            with torch.cuda.stream(stream):
+                for i in range(2 * copies):
+                    launch(bits, n, k, x, ring[i % copies], sc, zr, y)
+                stream.synchronize()
+            plans.append(f"{name} M={m}: " + _lib.describe_plan(bits, GROUP, n, k, m, True))
+        print(json.dumps({"counter_pass": plans, "launches_each": 32}))
         return 0
     if args.counter_pass:
         n, k = LLAMA3_8B["gate_up"]
