@@ -101,22 +101,22 @@ class Block(torch.nn.Module):
         self.input_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=dtype, device=device), requires_grad=False)
         self.post_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=dtype, device=device), requires_grad=False)
 
-    def forward(self, h, cos, sin, pos, k_cache, v_cache, mask):
+    def forward(self, h, cos, sin, pos, k_cache, v_cache, bias):
         """h [M, hidden]; cos/sin [M, head_dim]; pos int64 [M] (cache rows written);
-        k_cache/v_cache [kv_heads, ctx, head_dim]; mask bool [M, ctx] (True = attend)."""
+        k_cache/v_cache [kv_heads, ctx, head_dim]; bias [rep * M, ctx] (0 = attend, -inf = not),
+        rows ordered like the queries of one key/value head: query head major, batch row minor."""
         cfg = self.cfg
         m, d, rep = h.shape[0], cfg.head_dim, cfg.heads // cfg.kv_heads
         x = torch.nn.functional.rms_norm(h, (cfg.hidden,), self.input_norm, cfg.rms_eps)
         qkv = self.qkv(x).view(m, cfg.heads + 2 * cfg.kv_heads, d)
-        q, k, v = qkv[:, :cfg.heads], qkv[:, cfg.heads:cfg.heads + cfg.kv_heads], qkv[:, cfg.heads + cfg.kv_heads:]
-        q, k = _rotate(q, cos, sin), _rotate(k, cos, sin)
-        k_cache.index_copy_(1, pos, k.transpose(0, 1))
-        v_cache.index_copy_(1, pos, v.transpose(0, 1))
-        # grouped-query attention: the `rep` query heads of a key/value head share one batched product
-        qg = q.transpose(0, 1).reshape(cfg.kv_heads, rep * m, d)
-        scores = torch.bmm(qg, k_cache.transpose(1, 2)).float() * (d ** -0.5)  # [kv, rep*m, ctx]
-        scores = scores.view(cfg.kv_heads, rep, m, -1).masked_fill(~mask, float("-inf"))
-        probs = torch.softmax(scores, dim=-1).to(h.dtype).view(cfg.kv_heads, rep * m, -1)
+        qk = _rotate(qkv[:, :cfg.heads + cfg.kv_heads], cos, sin)  # queries and keys in one pass
+        k_cache.index_copy_(1, pos, qk[:, cfg.heads:].transpose(0, 1))
+        v_cache.index_copy_(1, pos, qkv[:, cfg.heads + cfg.kv_heads:].transpose(0, 1))
+        # grouped-query attention: the `rep` query heads of a key/value head share one batched
+        # product; the mask enters as the additive term of that product
+        qg = qk[:, :cfg.heads].transpose(0, 1).reshape(cfg.kv_heads, rep * m, d)
+        scores = torch.baddbmm(bias, qg, k_cache.transpose(1, 2), alpha=d ** -0.5)  # [kv, rep*m, ctx]
+        probs = torch.softmax(scores, dim=-1)  # (accumulates in fp32 internally)
         attn = torch.bmm(probs, v_cache).view(cfg.heads, m, d).transpose(0, 1).reshape(m, cfg.hidden)
         h = h + self.o(attn)
         x = torch.nn.functional.rms_norm(h, (cfg.hidden,), self.post_norm, cfg.rms_eps)
@@ -160,9 +160,10 @@ class Decoder(torch.nn.Module):
         """tokens int64 [M], pos int64 [M] (their positions) -> logits [M, vocab] (fp32)."""
         h = self.embed.index_select(0, tokens)
         cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
-        mask = self.arange[None, :] <= pos[:, None]
+        rep = self.cfg.heads // self.cfg.kv_heads
+        bias = torch.where(self.arange[None, :] <= pos[:, None], 0.0, float("-inf")).to(h.dtype).repeat(rep, 1)
         for i, block in enumerate(self.blocks):
-            h = block(h, cos, sin, pos, cache[i, 0], cache[i, 1], mask)
+            h = block(h, cos, sin, pos, cache[i, 0], cache[i, 1], bias)
         h = torch.nn.functional.rms_norm(h, (self.cfg.hidden,), self.final_norm, self.cfg.rms_eps)
         return torch.nn.functional.linear(h[-1:], self.head).float()
 
