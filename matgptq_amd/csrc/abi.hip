@@ -93,13 +93,15 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   }
   // default prefill tile (measured on MI355X, Llama-3-70B layers): 128 x 256 (two waves per
   // SIMD, activations copied straight into LDS) once its workgroups fill most of the 512
-  // resident slots; below that 128 x 128, and 32 x 128 while the batch is small
+  // resident slots; below that 128 x 128 when that tile still gives about 200 workgroups or
+  // the batch exceeds 512 rows, else 32 x 128
   if (!p->decode) {
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
     // (bf16 storage has no ring loop: its 128 x 256 tile runs one wave per SIMD)
+    const int64_t wgs_128 = ((N + 127) / 128) * ((M + 127) / 128);
     if (wgs_big >= 448 && !(flags & MATGPTQ_FLAG_BF16)) p->cfg = 0;
-    else if (M <= 512) p->cfg = 4;
-    else p->cfg = 3;
+    else if (M > 512 || (wgs_128 >= 200 && M >= 112)) p->cfg = 3;  // (a batch that fills most of a 128-row tile)
+    else p->cfg = 4;
     // Mid-batch kernel (K split inside the workgroup) against the 32 x 128 tile, as measured on
     // MI355X (4 bits, Llama-3-8B layers): the former dequantises every code once per 32 batch
     // rows, about 2 us + 0.13 us per million codes and batch tile; the latter walks K serially,

@@ -44,7 +44,10 @@ constexpr int kBits = MATGPTQ_BITS;
 constexpr int kWaves = 8;
 
 // Stages of a wave's ring: as many as fit 128 KB of LDS per workgroup.
-constexpr int skinny_stages(int mb) { return 4 / mb; }
+#ifndef MATGPTQ_EXP_NS1
+#define MATGPTQ_EXP_NS1 4
+#endif
+constexpr int skinny_stages(int mb) { return mb == 1 ? MATGPTQ_EXP_NS1 : 2; }
 
 // LDS of a workgroup: per wave and stage an activation buffer of 16*MB rows x 256 bytes; the
 // partial sums (16 bytes per lane, row block and batch block per wave) reuse them after the loop.
