@@ -114,13 +114,15 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       const double walk = 0.82 * k_tiles * (wgs > 512 ? (double)wgs / 512.0 : 1.0);
       p->skinny = mid < walk;
     }
-  } else if (flavour == 0 && row_blocks < 1024 &&
-             (M >= 8 || (M >= 4 && k_tiles >= 64) || (M >= 2 && k_tiles >= 112))) {
-    // Small batches of layers with few rows: every decode workgroup stages the whole batch of
-    // activations (scaled copies, written by the vector ALU), which grows with M and K, while
-    // the mid-batch kernel copies them into LDS asynchronously.  Measured on MI355X (Llama-3-8B
-    // and 70B layers, 3 and 4 bits): the latter wins from these batch sizes on; on the layers
-    // with many rows the decode kernel stays ahead up to M = 16.
+  } else if (flavour == 0 &&
+             (row_blocks < 1024 ? (M >= 8 || (M >= 4 && k_tiles >= 64) || (M >= 2 && k_tiles >= 112))
+                                : (M >= 8 && bits <= 6 && group_size != 32))) {
+    // Small batches: every decode workgroup stages the whole batch of activations (scaled
+    // copies, written by the vector ALU), which grows with M and K, while the mid-batch kernel
+    // copies them into LDS asynchronously.  Measured on MI355X (Llama-3-8B and 70B layers, 3 and
+    // 4 bits): the latter wins from eight batch rows on, and earlier on layers with few rows
+    // and a long K; on layers with many rows only where it may take four row blocks per
+    // workgroup (up to 6 bits, one scale per tile).
     p->decode = false;
     p->skinny = true;
     p->mb = 1;

@@ -17,11 +17,14 @@
 //    would touch sixteen rows with sixteen adjacent lanes).  16-byte chunk c of row r lies at
 //    position c ^ (r & 15) of the LDS row, so the sixteen lanes of an operand read hit sixteen
 //    different bank groups;
-//  * a wave keeps a ring of 4 / MB stages (an LDS buffer and a register set of codes, scales
-//    and zeros each) and requests a tile as many tiles ahead: a walk is short (K / 1024
-//    tiles), so what hides the memory latency is the depth of that ring, not a long loop.
-//    Only the wave itself waits for its copies (vmcnt, counted by hand: every stage issues the
-//    same number of instructions, so "all but the youngest stages" is a constant); there is no
+//  * a wave has one LDS buffer and two register sets of codes, scales and zeros.  At the start
+//    of a tile it waits for its own copies and loads (vmcnt(0): nothing younger is in flight),
+//    reads the tile's operands from LDS into registers, and only then requests the next tile
+//    into the same buffer and the other register set, which arrive while this tile is
+//    dequantised and multiplied.  One buffer instead of two keeps the LDS of a workgroup at
+//    32 KB per 16 batch rows, so that several workgroups share a CU: a walk is short (K / 1024
+//    tiles) and what hides the memory latency is the number of waves, not the depth of a
+//    ring (a four-deep ring at 128 KB per workgroup measured 10-30 % slower).  There is no
 //    barrier in the loop;
 //  * every load is branch-free (tiles beyond K, rows beyond M or N go through a zero-length
 //    buffer descriptor or an out-of-range offset);
@@ -44,15 +47,10 @@ constexpr int kBits = MATGPTQ_BITS;
 constexpr int kWaves = 8;
 
 // Stages of a wave's ring: as many as fit 128 KB of LDS per workgroup.
-#ifndef MATGPTQ_EXP_NS1
-#define MATGPTQ_EXP_NS1 4
-#endif
-constexpr int skinny_stages(int mb) { return mb == 1 ? MATGPTQ_EXP_NS1 : 2; }
-
-// LDS of a workgroup: per wave and stage an activation buffer of 16*MB rows x 256 bytes; the
-// partial sums (16 bytes per lane, row block and batch block per wave) reuse them after the loop.
+// LDS of a workgroup: per wave one activation buffer of 16*MB rows x 256 bytes; the partial
+// sums (16 bytes per lane, row block and batch block per wave) reuse them after the loop.
 constexpr int skinny_lds_bytes(int r, int mb) {
-  const int stage = kWaves * skinny_stages(mb) * mb * 16 * 256, sums = kWaves * r * mb * 64 * 16;
+  const int stage = kWaves * mb * 16 * 256, sums = kWaves * r * mb * 64 * 16;
   return stage > sums ? stage : sums;
 }
 
@@ -61,10 +59,8 @@ __global__ void __launch_bounds__(64 * kWaves, 2)
 skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   constexpr int GPT = GROUP == 32 ? 4 : 1;
   constexpr int kStage = MB * 16 * 256;  // bytes of one activation buffer
-  constexpr int NS = skinny_stages(MB);  // stages of the ring; a tile is requested NS - 1 tiles ahead
-  // vector-memory instructions of one stage: activation copies, then codes, scales, zeros
-  constexpr int kIssue = 4 * MB + R * (tile_load_count(BITS) + GPT * (ZP ? 2 : 1));
-  __shared__ __align__(16) unsigned char smem[skinny_lds_bytes(R, MB)];  // (this target has 160 KB per workgroup)
+  constexpr int NS = 2;  // register sets of codes, scales, zeros
+  __shared__ __align__(16) unsigned char smem[skinny_lds_bytes(R, MB)];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -121,7 +117,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 
   // Copy of one tile's activations: instruction i moves rows 4i .. 4i+3 (lane l: row 4i + l/16,
   // LDS position l%16, which holds chunk (l%16) ^ (row & 15) of the row's 256 bytes).
-  unsigned char* const stage = smem + wave * (NS * kStage);
+  unsigned char* const stage = smem + wave * kStage;
   uint32_t dma_voff[4 * MB];
 #pragma unroll
   for (int i = 0; i < 4 * MB; i++) {
@@ -130,20 +126,18 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     const uint32_t m = (uint32_t)(m0 + row);
     dma_voff[i] = m < (uint32_t)a.M ? m * (uint32_t)a.K * 2u + c * 16 : x_bytes;
   }
-  auto dma = [&](int buf, int kb) {
+  auto dma = [&](int kb) {
     const BufRsrc xres = make_rsrc(a.x, kb < a.k_tiles ? x_bytes : 0u);
 #pragma unroll
     for (int i = 0; i < 4 * MB; i++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          xres, (__attribute__((address_space(3))) void*)(stage + buf * kStage + i * 1024), 16, (int)dma_voff[i],
+          xres, (__attribute__((address_space(3))) void*)(stage + i * 1024), 16, (int)dma_voff[i],
           (int)((uint32_t)kb * 256u), 0, 0);  // (int: the builtin's own parameter type)
     __builtin_amdgcn_sched_barrier(0);
   };
   // operand of batch rows i*16 + r16, columns [j*32 + q*8, +8) of the tile: chunk 4j + q
-  auto read_frag = [&](int buf, int i, int j) {
-    const half8 raw = *reinterpret_cast<const half8*>(stage + buf * kStage + (i * 16 + r16) * 256 +
-                                                      (((4 * j + q) ^ r16) * 16));
-    return storage8_to_half8(raw);
+  auto read_frag = [&](int i, int j) {
+    return *reinterpret_cast<const half8*>(stage + (i * 16 + r16) * 256 + (((4 * j + q) ^ r16) * 16));
   };
 
   auto dequant_step = [&](Frag (&aw)[R], const uint32_t (&w)[R][BITS], const uint32_t (&s)[R][GPT],
@@ -169,24 +163,26 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     }
   };
 
-  // Tile t of the walk (K tile kb = wave + 8 t) lives in stage t % NS (`btag`).  Stages are
-  // issued in tile order, NS - 1 tiles ahead, kIssue instructions each: at the start of tile t
-  // everything up to stage t must have arrived and the NS - 2 younger stages may be in flight.
-  auto issue = [&](auto btag, int kb) {
-    constexpr int B = decltype(btag)::value;
-    dma(B, kb);
-    load_weights(wr[B], sr[B], zr[B], kb);
-  };
+  // Tile t of the walk (K tile kb = wave + 8 t), codes in register set `btag`.
   auto tile = [&](int t, auto btag) {
     constexpr int B = decltype(btag)::value;
     const int kb = wave + t * kWaves;
-    // (the counter holds 63 at most: waiting for fewer in flight than necessary is safe)
-    constexpr int n = (NS - 2) * kIssue < 63 ? (NS - 2) * kIssue : 63;
+    // everything this wave has requested has arrived: the copy of this tile's activations and
+    // this tile's codes were the last requests
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt((n & 15) | (7 << 4) | (0 << 8) | ((n >> 4) << 14));  // vmcnt(n), lgkmcnt(0)
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (0 << 8) | (0 << 14));  // vmcnt(0), lgkmcnt(0)
     __builtin_amdgcn_sched_barrier(0);
-    // the stage of tile t - 1 is free: its operands have been read, its codes dequantised
-    issue(std::integral_constant<int, (B + NS - 1) % NS>{}, kb + (NS - 1) * kWaves);
+    half8 xf[4][MB];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < MB; i++) xf[j][i] = read_frag(i, j);
+    // the buffer is free once these reads have returned: request the next tile
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14));  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    dma(kb + kWaves);
+    load_weights(wr[B ^ 1], sr[B ^ 1], zr[B ^ 1], kb + kWaves);
     if (kb < a.k_tiles) {
       auto one = [&](auto jtag) {
         constexpr int J = decltype(jtag)::value;
@@ -194,7 +190,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
         dequant_step(aw, wr[B], sr[B], zr[B], jtag);
 #pragma unroll
         for (int i = 0; i < MB; i++) {
-          const half8 b = read_frag(B, i, J);
+          const half8 b = storage8_to_half8(xf[J][i]);
 #pragma unroll
           for (int rr = 0; rr < R; rr++)
             acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b, acc[rr][i], 0, 0, 0);
@@ -205,24 +201,16 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
       one(std::integral_constant<int, 2>{});
       one(std::integral_constant<int, 3>{});
     }
-    // (the next tile's wait must not move above this tile's operand reads)
     __builtin_amdgcn_sched_barrier(0);
   };
 
   const int walk = (a.k_tiles + kWaves - 1) / kWaves;  // tiles of the longest walk
   __builtin_amdgcn_sched_barrier(0);
-  issue(std::integral_constant<int, 0>{}, wave);
-  if constexpr (NS == 4) {
-    issue(std::integral_constant<int, 1>{}, wave + kWaves);
-    issue(std::integral_constant<int, 2>{}, wave + 2 * kWaves);
-  }
-  for (int t = 0; t < walk; t += NS) {
+  dma(wave);
+  load_weights(wr[0], sr[0], zr[0], wave);
+  for (int t = 0; t < walk; t += 2) {
     tile(t, std::integral_constant<int, 0>{});
     tile(t + 1, std::integral_constant<int, 1>{});
-    if constexpr (NS == 4) {
-      tile(t + 2, std::integral_constant<int, 2>{});
-      tile(t + 3, std::integral_constant<int, 3>{});
-    }
   }
 
   // The eight partial sums of every output meet in LDS (over the activation buffers: every

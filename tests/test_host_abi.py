@@ -129,7 +129,9 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(4, 128, 4096, 4096, 1).startswith("decode")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048).startswith("prefill")
     assert _lib.describe_plan(4, 128, 4096, 4096, 4, True).startswith("decode")
-    assert _lib.describe_plan(4, 128, 28672, 4096, 16, True).startswith("decode")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 4, True).startswith("decode")
+    assert _lib.describe_plan(8, 128, 28672, 4096, 16, True).startswith("decode")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 16, True) == "midbatch b4 g128 zp1 R4 mb1"
     # small layers: the mid-batch kernel (K split inside the workgroup) from a few rows on
     assert _lib.describe_plan(4, 128, 4096, 4096, 8, True).startswith("midbatch")
     assert _lib.describe_plan(4, 128, 4096, 14336, 2, True).startswith("midbatch")
