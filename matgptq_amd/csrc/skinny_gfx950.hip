@@ -1,4 +1,5 @@
-// Mid-batch kernel (16 < M <= a few hundred): the K dimension is split inside the workgroup.
+// Mid-batch kernel (a few batch rows up to a few hundred): the K dimension is split inside the
+// workgroup.
 // Compiled once per bitwidth with -DMATGPTQ_BITS=b.
 //
 // At these batch sizes a layer has few output tiles: a kernel that gives every workgroup a
@@ -12,8 +13,8 @@
 //  * each wave dequantises its tiles from registers into the 16x32 MFMA operand (the same
 //    arithmetic as the large-batch kernel).  No two waves of a workgroup read the same
 //    activations, so every wave stages its own: buffer_load ... lds copies the 16*MB x 128
-//    activations of a tile from global memory straight into one of the wave's private LDS
-//    buffers, 256 contiguous bytes per 16 lanes (an operand read straight from global memory
+//    activations of a tile from global memory straight into the wave's private LDS buffer,
+//    256 contiguous bytes per 16 lanes (an operand read straight from global memory
 //    would touch sixteen rows with sixteen adjacent lanes).  16-byte chunk c of row r lies at
 //    position c ^ (r & 15) of the LDS row, so the sixteen lanes of an operand read hit sixteen
 //    different bank groups;
@@ -90,8 +91,8 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     for (int i = 0; i < MB; i++) acc[rr][i] = float4v{0.f, 0.f, 0.f, 0.f};
 
   const UnpackConsts<BITS> kc_unpack;
-  // codes, scales and zeros of every stage; scales and zeros stay as loaded and are converted
-  // where they are used
+  // codes, scales and zeros of the tile in use and of the next one; scales and zeros stay as
+  // loaded and are converted where they are used
   uint32_t wr[NS][R][BITS], sr[NS][R][GPT], zr[NS][R][GPT];
 
   auto load_weights = [&](uint32_t (&w)[R][BITS], uint32_t (&s)[R][GPT], uint32_t (&z)[R][GPT], int kb) {
