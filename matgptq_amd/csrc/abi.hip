@@ -67,7 +67,7 @@ size_t decode_lds_bytes(int R, int S, int W, int kc, int64_t M) {
 // Automatic choice; the flags word can override it for benchmarks:
 //   bits 8..15 : 0 = automatic, 1 + rsel + 3*shape = decode (rsel: R = 1,2,4; shape: kShapes),
 //                64 + cfg = prefill tile configuration,
-//                80 + rsel + 3*(mb-1) = mid-batch kernel (rsel: R = 1,2,4; mb: 16 or 32 batch rows)
+//                80 + rsel + 3*msel = mid-batch kernel (rsel: R = 1,2,4; msel: 16, 32, 64 batch rows)
 //   bits 16..17: decode flavour, 0 = automatic, 1 = burst, 2 = stream
 int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp, uint32_t flags,
               Plan* p) {
@@ -91,57 +91,74 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     if (row_blocks >= 1024) { R = 2; S = 2; W = 4; }
     else if (row_blocks >= 320) { R = 2; }
   }
-  // default prefill tile (measured on MI355X, Llama-3-70B layers): 128 x 256 (two waves per
-  // SIMD, activations copied straight into LDS) once its workgroups fill most of the 512
-  // resident slots; below that 128 x 128 when that tile still gives about 200 workgroups or
-  // the batch exceeds 512 rows, else 32 x 128
+  // (four row blocks per mid-batch workgroup only up to 6 bits and one scale per tile: registers)
+  const int r_max = group_size == 32 || bits > 6 ? 2 : 4;
+  // row blocks per mid-batch workgroup: as many as still leave about 160 workgroups (the
+  // activations are re-read once per workgroup column)
+  auto mid_rows = [&](int64_t m_tiles) {
+    for (int r = r_max; r > 1; r >>= 1)
+      if ((int64_t)((row_blocks + r - 1) / r) * m_tiles >= 160) return r;
+    return 1;
+  };
   if (!p->decode) {
+    // M > 16.  The 128 x 256 tile (two waves per SIMD, activations copied straight into LDS)
+    // once its workgroups fill most of the 512 resident slots (measured on MI355X, Llama-3-70B
+    // layers; bf16 storage has no ring loop, its 128 x 256 tile runs one wave per SIMD).
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
-    // (bf16 storage has no ring loop: its 128 x 256 tile runs one wave per SIMD)
-    const int64_t wgs_128 = ((N + 127) / 128) * ((M + 127) / 128);
-    if (wgs_big >= 448 && !(flags & MATGPTQ_FLAG_BF16)) p->cfg = 0;
-    else if (M > 512 || (wgs_128 >= 200 && M >= 112)) p->cfg = 3;  // (a batch that fills most of a 128-row tile)
-    else p->cfg = 4;
-    // Mid-batch kernel (K split inside the workgroup) against the 32 x 128 tile, as measured on
-    // MI355X (4 bits, Llama-3-8B layers): the former dequantises every code once per 32 batch
-    // rows, about 2 us + 0.13 us per million codes and batch tile; the latter walks K serially,
-    // about 0.82 us per K tile while its workgroups fit the 512 resident slots and
-    // proportionally more beyond.
-    if (p->cfg == 4) {
-      const int64_t m_tiles = (M + 31) / 32;
-      const double mid = 2.0 + 0.13e-6 * (double)m_tiles * (double)N * (double)K;
-      const int64_t wgs = ((N + 127) / 128) * m_tiles;
-      const double walk = 0.82 * k_tiles * (wgs > 512 ? (double)wgs / 512.0 : 1.0);
-      p->skinny = mid < walk;
+    if (wgs_big >= 448 && !(flags & MATGPTQ_FLAG_BF16)) {
+      p->cfg = 0;
+    } else {
+      // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
+      // (4 bits, Llama-3-8B and 70B layers, M = 17 .. 1024), in microseconds:
+      //   128 x 128 tile  1.33 per K tile, up to 1.5 times that as a second workgroup joins a CU,
+      //                   proportionally more beyond the 512 resident slots;
+      //   32 x 128 tile   0.95 per K tile, proportionally more beyond 512 workgroups;
+      //   mid-batch kernel with 32 or 64 batch rows per workgroup: 2 + rounds x K tiles x
+      //                   (0.12 + 0.016 R MB), one workgroup per CU and round when its registers or
+      //                   LDS allow no second one (R = 4 or MB = 4), else two.
+      const double kt = (double)k_tiles;
+      const int64_t wgs_128 = ((N + 127) / 128) * ((M + 127) / 128);
+      const int64_t wgs_32 = ((N + 127) / 128) * ((M + 31) / 32);
+      const double second = wgs_128 <= 256 ? 0.0 : wgs_128 >= 512 ? 1.0 : (double)(wgs_128 - 256) / 256.0;
+      const double t_128 = 1.33 * kt * (1.0 + 0.5 * second) * (wgs_128 > 512 ? (double)wgs_128 / 512.0 : 1.0);
+      const double t_32 = 0.95 * kt * (wgs_32 > 512 ? (double)wgs_32 / 512.0 : 1.0);
+      p->cfg = t_128 < t_32 ? 3 : 4;
+      double best = t_128 < t_32 ? t_128 : t_32;
+      for (int mb = 2; mb <= (M > 32 ? 4 : 2); mb <<= 1) {
+        const int64_t m_tiles = (M + 16 * mb - 1) / (16 * mb);
+        const int r = mid_rows(m_tiles);
+        const int64_t wgs = (int64_t)((row_blocks + r - 1) / r) * m_tiles;
+        const int64_t slots = 256 * (mb == 4 || r == 4 ? 1 : 2);
+        const double t = 2.0 + (double)((wgs + slots - 1) / slots) * kt * (0.12 + 0.016 * r * mb);
+        if (t < best) {
+          best = t;
+          p->skinny = true;
+          p->mb = mb;
+          R = r;
+        }
+      }
     }
   } else if (flavour == 0 &&
              (row_blocks < 1024 ? (M >= 8 || (M >= 4 && k_tiles >= 64) || (M >= 2 && k_tiles >= 112))
-                                : (M >= 8 && bits <= 6 && group_size != 32))) {
+                                : (M >= 8 && r_max == 4))) {
     // Small batches: every decode workgroup stages the whole batch of activations (scaled
     // copies, written by the vector ALU), which grows with M and K, while the mid-batch kernel
     // copies them into LDS asynchronously.  Measured on MI355X (Llama-3-8B and 70B layers, 3 and
     // 4 bits): the latter wins from eight batch rows on, and earlier on layers with few rows
     // and a long K; on layers with many rows only where it may take four row blocks per
-    // workgroup (up to 6 bits, one scale per tile).
+    // workgroup.
     p->decode = false;
     p->skinny = true;
     p->mb = 1;
-  }
-  if (p->skinny) {
-    // as many row blocks per workgroup as still leave about 160 workgroups (the activations
-    // are re-read once per workgroup column)
-    const int64_t m_tiles = (M + 16 * p->mb - 1) / (16 * p->mb);
-    R = 1;
-    for (int r = 4; r > 1; r >>= 1)
-      if ((int64_t)((row_blocks + r - 1) / r) * m_tiles >= 160) { R = r; break; }
+    R = mid_rows(1);
   }
   if (variant != 0) {
     if (variant >= 80) {
-      if (variant - 80 > 5) return MATGPTQ_EVARIANT;
+      if (variant - 80 > 8) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->skinny = true;
       R = 1 << ((variant - 80) % 3);
-      p->mb = 1 + (variant - 80) / 3;
+      p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
       if (variant - 64 > 7) return MATGPTQ_EVARIANT;
       p->decode = false;
@@ -163,8 +180,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     // the prefill kernel addresses X through a 32-bit buffer offset
     if ((uint64_t)M * (uint64_t)K * 2u >= (1ull << 32)) return MATGPTQ_ESIZE;
     p->R = p->S = p->W = p->kc = 0;
-    // (four row blocks per workgroup only up to 6 bits and one scale per tile: register budget)
-    if (p->skinny) p->R = R >= 4 && (group_size == 32 || bits > 6) ? 2 : R;
+    if (p->skinny) p->R = R > r_max ? r_max : R;  // (a forced variant may ask for more)
     p->stream = false;
     p->smem = 0;
     return MATGPTQ_OK;

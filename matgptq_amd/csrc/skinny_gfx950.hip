@@ -264,6 +264,7 @@ hipError_t launch_rows(const GemmArgs& a, int r, hipStream_t s) {
 
 template <int GROUP, bool ZP>
 hipError_t launch_batch(const GemmArgs& a, int r, int mb, hipStream_t s) {
+  if (mb >= 4) return launch_rows<GROUP, ZP, 4>(a, r, s);
   return mb >= 2 ? launch_rows<GROUP, ZP, 2>(a, r, s) : launch_rows<GROUP, ZP, 1>(a, r, s);
 }
 

@@ -141,7 +141,7 @@ def test_midbatch_kernel_every_format(b, g, zp):
     n, k, m = 304, 128 * 13, 77
     lay = G.Layer(n, k, b, g, seed=17 * b + (g & 7), zero_points=zp)
     x = o.make_activations(m, k, seed=b + 1)
-    for rsel in range(6):
+    for rsel in range(9):
         flags = 1 | ((80 + rsel) << 8)
         y = lay.run(x, flags=flags)
         G.assert_close_to_oracle(y, x, lay.w, f"mid-batch b={b} g={g} zp={zp} rsel={rsel}")
@@ -155,7 +155,7 @@ def test_midbatch_kernel_shapes(n, k, m):
     lay = G.Layer(n, k, 4, 128, seed=n + m)
     x = o.make_activations(m, k, seed=m)
     rows = np.r_[0:min(m, 24), max(m - 24, 0):m]
-    for rsel in range(6):
+    for rsel in range(9):
         y = lay.run(x, flags=1 | ((80 + rsel) << 8))
         G.assert_close_to_oracle(y[rows], x[rows], lay.w, f"mid-batch {n}x{k} M={m} rsel={rsel}")
 
@@ -176,7 +176,7 @@ def test_midbatch_kernel_agrees_with_prefill_tile_closely():
 def test_midbatch_kernel_outlier_channels():
     lay = G.Layer(512, 4096, 3, 128, seed=12)
     x = o.make_activations(48, 4096, seed=3, outlier_frac=0.01, outlier_gain=20.0)
-    for rsel in range(6):
+    for rsel in range(9):
         G.assert_close_to_oracle(lay.run(x, flags=1 | ((80 + rsel) << 8)), x, lay.w, f"outliers rsel={rsel}")
 
 
@@ -386,7 +386,7 @@ def test_bf16_midbatch_kernel(b, g, zp):
     x = o.round_to_bf16(o.make_activations(m, k, seed=9).astype(np.float32))
     pk = G.pack_device(q, b, True)
     ref = o.linear_f64(x, o.dequantize_bf16(q, s, z, b, g))
-    for rsel in range(6):
+    for rsel in range(9):
         y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | ((80 + rsel) << 8))
         assert np.all(np.isfinite(y))
         assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref)), (b, g, zp, rsel)
