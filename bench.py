@@ -362,6 +362,21 @@ def cpu_path_baseline(step_bytes: int):
             for q, s, z, x in layers:
                 torch_path.forward(x, q, s, z, 8, 4)
             best = min(best, time.perf_counter() - t0)
+        # the matrix product alone on weights dequantised beforehand, fp16 and fp32 (CPU fp16
+        # GEMV can be much slower than fp32: both are stated)
+        ws = [torch_path.get_weight(q, s, z, 8, 4) for q, s, z, _ in layers]
+        only = {}
+        for tag, cast in (("fp16", lambda t: t), ("fp32", lambda t: t.float())):
+            wl = [cast(w) for w in ws]
+            xl = [cast(x) for _, _, _, x in layers]
+            torch.nn.functional.linear(xl[1], wl[1])
+            t_best = float("inf")
+            for _ in range(5):
+                t0 = time.perf_counter()
+                for w, x in zip(wl, xl):
+                    torch.nn.functional.linear(x, w)
+                t_best = min(t_best, time.perf_counter() - t0)
+            only[tag] = t_best
     return {
         "value": round(step_bytes / best / 1e9, 3),
         "unit": "GB/s",
@@ -369,6 +384,7 @@ def cpu_path_baseline(step_bytes: int):
         "kind": "port",
         "sample": f"one full step (4 layers, M=1, 4-bit), best of 5, {best:.3f} s per step: "
                   "slice + dequantize + F.linear in torch on the host, fp16",
+        "linear_only_s_per_step": {k: round(v, 4) for k, v in only.items()},
     }
 
 
