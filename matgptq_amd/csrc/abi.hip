@@ -102,10 +102,10 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   };
   if (!p->decode) {
     // M > 16.  The 128 x 256 tile (two waves per SIMD, activations copied straight into LDS)
-    // once its workgroups fill most of the 512 resident slots (measured on MI355X, Llama-3-70B
-    // layers; bf16 storage has no ring loop, its 128 x 256 tile runs one wave per SIMD).
+    // once its workgroups fill more than half of the 512 resident slots (measured on MI355X,
+    // Llama-3-8B and 70B layers; bf16 storage has no ring loop, its 128 x 256 tile runs one wave per SIMD).
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
-    if (wgs_big >= 448 && !(flags & MATGPTQ_FLAG_BF16)) {
+    if (wgs_big >= 288 && !(flags & MATGPTQ_FLAG_BF16)) {
       p->cfg = 0;
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
