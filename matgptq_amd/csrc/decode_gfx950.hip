@@ -14,8 +14,9 @@
 //
 // Arithmetic.  The VALU only masks the codes into "raw" fp16 pairs
 // 1024 + c*2^p (one v_and_or_b32 / v_perm_b32 per two codes).  Everything else
-// runs on the matrix cores, with fp32 accumulation, on X' = X * 2^-p staged once
-// per workgroup in LDS (p depends only on the position inside an octet):
+// runs on the matrix cores, with fp32 accumulation, on X' = X * 2^-p staged in LDS
+// (p depends only on the position inside an octet; once per workgroup for M > 1, while at
+// M = 1 every wave stages just the columns of its own tiles and starts without a barrier):
 //     D += raw        * X'      ->  sum (1024*2^-p + c) x
 //     D -= (1024 + 2^(b-1) 2^p) * X'   (constant operand)  ->  sum (c - 2^(b-1)) x
 //     D -= (zero-128)/2^(8-b) 2^p * X' (one value per row and group, zero-point form only)
@@ -371,18 +372,41 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
     }
   };
 
+  // M = 1: a wave reads only the activations of its own tiles (ws, ws + W, ...), so it stages
+  // exactly those, 16 chunks per tile, and needs no barrier before it starts: trip j covers the
+  // wave's tiles 4 XU j .. 4 XU (j+1) - 1, lane l the chunk l % 16 of tile 4 (XU j + i) + l / 16.
+  // A tile beyond K repeats the wave's first tile (same value to the same place).
+  auto x_fetch_own = [&](XTrip& t, int j) {
+    const half8* src = reinterpret_cast<const half8*>(a.x);
+#pragma unroll
+    for (int i = 0; i < XU; i++) {
+      const int ti = ws + W * (4 * (XU * j + i) + q);
+      const int c = (ti < a.k_tiles ? ti : ws) * 16 + r16;
+      t.dst[i] = c * 8;
+      t.odd[i] = BITS == 2 && ((c >> 2) & 1) != 0;
+      t.v[i] = src[c];
+    }
+  };
+
   XTrip xt;
   if constexpr (!CHUNKED) {
     // all of X' fits in LDS
     const int n_stages = stages_of(0, a.k_tiles);
-#ifndef MATGPTQ_DEBUG_NOSTAGE
-    x_fetch(xt, 0, a.k_tiles * 16, tid);
-#endif
-    load_stage(cur, 0, a.k_tiles, 0);
-#ifndef MATGPTQ_DEBUG_NOSTAGE
-    stage_x(xt, 0, a.k_tiles);
-    __syncthreads();
-#endif
+    if (a.M == 1) {
+      x_fetch_own(xt, 0);
+      load_stage(cur, 0, a.k_tiles, 0);
+      x_commit(xt);
+      const int own = (a.k_tiles - ws + W - 1) / W;  // (W <= K / 128: every wave has a tile)
+      for (int j = 1; j * 4 * XU < own; j++) {
+        x_fetch_own(xt, j);
+        x_commit(xt);
+      }
+    } else {
+      x_fetch(xt, 0, a.k_tiles * 16, tid);
+      load_stage(cur, 0, a.k_tiles, 0);
+      stage_x(xt, 0, a.k_tiles);
+      __syncthreads();
+    }
     run_stages(0, a.k_tiles, n_stages);
   } else {
     // K is walked in chunks of kc tiles so that the LDS copy of X' stays small
