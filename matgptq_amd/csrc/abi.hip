@@ -107,6 +107,13 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
     if (wgs_big >= 288 && !(flags & MATGPTQ_FLAG_BF16)) {
       p->cfg = 0;
+      // Whole rounds of 512 resident workgroups plus at most half a round: the rows of that
+      // fraction go to 128 x 128 tiles, which run last, one per CU, in about a third of a
+      // round's time (Llama-3-70B qkv at M = 2048, 640 tiles: 355 -> 305 us).
+      const int m_tiles = (int)((M + 127) / 128);
+      const int nb = prefill_tail_big_tiles(row_blocks, m_tiles);
+      const int64_t rest = (int64_t)((row_blocks - nb * 16 + 15) / 16) * m_tiles;
+      if (nb > 0 && rest > 0 && rest <= 256) p->cfg = 8;
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
       // (4 bits, Llama-3-8B and 70B layers, M = 17 .. 1024), in microseconds:
@@ -160,7 +167,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       R = 1 << ((variant - 80) % 3);
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
-      if (variant - 64 > 7) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 8) return MATGPTQ_EVARIANT;
+      if (variant - 64 == 8 && (flags & MATGPTQ_FLAG_BF16)) return MATGPTQ_EVARIANT;  // ring loop: fp16 storage only
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 64;

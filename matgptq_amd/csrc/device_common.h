@@ -333,4 +333,15 @@ struct GemmArgs {
   int row_blocks;           // N / 16
 };
 
+// Prefill with a tail of narrower tiles: how many 256-row weight tiles (of `row_blocks / 16` whole
+// ones) the 128 x 256 workgroups take before the 128 x 128 workgroups take the remaining rows -
+// the whole rounds of 512 resident workgroups (two per CU), in whole columns of `m_tiles`
+// activation tiles.
+inline int prefill_tail_big_tiles(int row_blocks, int m_tiles) {
+  const int n_tiles = row_blocks / 16;
+  const int per_round = 512 / m_tiles;  // weight tiles one round covers
+  if (per_round == 0) return n_tiles;
+  return n_tiles / per_round * per_round;
+}
+
 }  // namespace matgptq

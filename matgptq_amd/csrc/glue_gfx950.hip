@@ -1,0 +1,269 @@
+// The operators between the bit-sliced linears of a decoder block at decode time, fused so that
+// a block is nine launches: residual add + RMS norm, rotary embedding + cache write, attention
+// of a few query rows over a static key/value cache, SiLU gate.  They belong to the end-to-end
+// decode measurement (the reference leaves these operators to transformers / vLLM,
+// inference_lib/inference_demo_transformers.py:134-176, inference_lib/bench_transformers_e2e.py:61-76)
+// and are built into a library of their own, apart from the GEMM's C ABI.  fp16 storage, fp32
+// arithmetic.  All of them are small and latency-bound: one workgroup per row / head.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/matgptq_glue.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+// sum / maximum over the 256 threads of a workgroup; `red` holds 4 floats and is reused, so the
+// leading barrier keeps a later call from overwriting values an earlier one is still reading
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// h += delta (if given); x = h * rsqrt(mean(h^2) + eps) * weight.  One workgroup per row; a thread
+// keeps its chunks of the row in registers (H <= 8 * 256 * kMaxChunks).
+constexpr int kMaxChunks = 4;
+__global__ void __launch_bounds__(kThreads)
+add_rmsnorm_kernel(_Float16* __restrict__ h, const _Float16* __restrict__ delta,
+                   const _Float16* __restrict__ weight, _Float16* __restrict__ x, int H, float eps) {
+  __shared__ float red[4];
+  const int chunks = H / 8;
+  half8* hr = reinterpret_cast<half8*>(h + (size_t)blockIdx.x * H);
+  const half8* dr = delta ? reinterpret_cast<const half8*>(delta + (size_t)blockIdx.x * H) : nullptr;
+  half8 v[kMaxChunks];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; i++) {
+    const int c = threadIdx.x + i * kThreads;
+    if (c < chunks) {
+      v[i] = hr[c];
+      if (dr) {
+        v[i] = v[i] + dr[c];  // one fp16 rounding, like the residual add it replaces
+        hr[c] = v[i];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e++) ss += (float)v[i][e] * (float)v[i][e];
+    }
+  }
+  const float rs = rsqrtf(block_sum(ss, red) / (float)H + eps);
+  half8* xr = reinterpret_cast<half8*>(x + (size_t)blockIdx.x * H);
+  const half8* wr = reinterpret_cast<const half8*>(weight);
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; i++) {
+    const int c = threadIdx.x + i * kThreads;
+    if (c < chunks) {
+      const half8 w = wr[c];
+      half8 o;
+#pragma unroll
+      for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)v[i][e] * rs * (float)w[e]);
+      xr[c] = o;
+    }
+  }
+}
+
+// Rotary embedding (half-split pairs) of the query and key heads of one row of the fused qkv
+// output; queries are rotated in place, rotated keys and the values go to row pos[m] of the
+// caches [kv_heads, max_ctx, d].  Grid (heads + 2 kv_heads, M), 64 threads.
+__global__ void __launch_bounds__(64)
+rope_cache_kernel(_Float16* __restrict__ qkv, const _Float16* __restrict__ cos_t,
+                  const _Float16* __restrict__ sin_t, const int64_t* __restrict__ pos,
+                  _Float16* __restrict__ k_cache, _Float16* __restrict__ v_cache, int heads, int kv_heads,
+                  int d, int64_t max_ctx) {
+  const int head = blockIdx.x, m = blockIdx.y;
+  int64_t p = pos[m];
+  p = p < 0 ? 0 : (p >= max_ctx ? max_ctx - 1 : p);  // never outside the tables and caches
+  _Float16* src = qkv + ((size_t)m * (heads + 2 * kv_heads) + head) * d;
+  if (head >= heads + kv_heads) {
+    _Float16* dst = v_cache + ((size_t)(head - heads - kv_heads) * max_ctx + p) * d;
+    for (int i = threadIdx.x; i < d; i += 64) dst[i] = src[i];
+    return;
+  }
+  _Float16* dst = head < heads ? src : k_cache + ((size_t)(head - heads) * max_ctx + p) * d;
+  const _Float16* c = cos_t + (size_t)p * d;
+  const _Float16* s = sin_t + (size_t)p * d;
+  const int half = d / 2;
+  for (int i = threadIdx.x; i < half; i += 64) {
+    const float a = (float)src[i], b = (float)src[i + half];
+    const float lo = a * (float)c[i] - b * (float)s[i];
+    const float hi = b * (float)c[i + half] + a * (float)s[i + half];
+    dst[i] = (_Float16)lo;
+    dst[i + half] = (_Float16)hi;
+  }
+}
+
+// Attention of one query head of one row over the cache positions 0 .. pos[m] (head dimension
+// 128).  Sixteen lanes share a cache row (16 bytes each), sixteen rows per step of the workgroup;
+// the scores wait in LDS for the softmax, then the same walk accumulates the values.
+// Grid (heads, M), 256 threads, dynamic LDS: max_ctx floats + 16 x 128 floats + 4.
+__global__ void __launch_bounds__(kThreads)
+attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ k_cache,
+                 const _Float16* __restrict__ v_cache, const int64_t* __restrict__ pos,
+                 _Float16* __restrict__ out, int heads, int kv_heads, int64_t max_ctx, float scale) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr int d = 128;
+  float* scores = lds;                 // [max_ctx]
+  float* part = lds + max_ctx;         // [16][128]
+  float* red = part + 16 * d;          // [4]
+  const int head = blockIdx.x, m = blockIdx.y;
+  const int kvh = head / (heads / kv_heads);
+  int64_t p = pos[m];
+  p = p < 0 ? 0 : (p >= max_ctx ? max_ctx - 1 : p);
+  const int n = (int)p + 1;
+  const int sub = threadIdx.x & 15, grp = threadIdx.x >> 4;
+
+  const half8 qv = *reinterpret_cast<const half8*>(qkv + ((size_t)m * (heads + 2 * kv_heads) + head) * d + sub * 8);
+  float q[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) q[e] = (float)qv[e] * scale;
+  const _Float16* kb = k_cache + (size_t)kvh * max_ctx * d + sub * 8;
+  const _Float16* vb = v_cache + (size_t)kvh * max_ctx * d + sub * 8;
+
+  float mx = -INFINITY;
+  for (int t = grp; t < n; t += 16) {
+    const half8 kv = *reinterpret_cast<const half8*>(kb + (size_t)t * d);
+    float dot = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) dot += q[e] * (float)kv[e];
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);  // the 16 lanes of a row are adjacent
+    if (sub == 0) scores[t] = dot;
+    mx = fmaxf(mx, dot);
+  }
+  mx = block_max(mx, red);  // (its barriers also publish the scores)
+  float sum = 0.f;
+  for (int t = threadIdx.x; t < n; t += kThreads) {
+    const float e = __expf(scores[t] - mx);
+    scores[t] = e;
+    sum += e;
+  }
+  sum = block_sum(sum, red);
+
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int t = grp; t < n; t += 16) {
+    const float pr = scores[t];
+    const half8 vv = *reinterpret_cast<const half8*>(vb + (size_t)t * d);
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] += pr * (float)vv[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) part[grp * d + sub * 8 + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < d) {
+    float o = 0.f;
+#pragma unroll
+    for (int g = 0; g < 16; g++) o += part[g * d + threadIdx.x];
+    out[((size_t)m * heads + head) * d + threadIdx.x] = (_Float16)(o / sum);
+  }
+}
+
+// out[m, j] = silu(gu[m, j]) * gu[m, F + j]; both factors rounded to fp16 like the two
+// element-wise operators it replaces.
+__global__ void __launch_bounds__(kThreads)
+silu_mul_kernel(const _Float16* __restrict__ gu, _Float16* __restrict__ out, int64_t M, int64_t F) {
+  const int64_t per_row = F / 8;
+  const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (c >= M * per_row) return;
+  const int64_t m = c / per_row, j = c - m * per_row;
+  const half8 g = *reinterpret_cast<const half8*>(gu + m * 2 * F + j * 8);
+  const half8 u = *reinterpret_cast<const half8*>(gu + m * 2 * F + F + j * 8);
+  half8 o;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    const float x = (float)g[e];
+    const _Float16 s = (_Float16)(x / (1.0f + __expf(-x)));
+    o[e] = s * u[e];
+  }
+  *reinterpret_cast<half8*>(out + m * F + j * 8) = o;
+}
+
+int launch_status() { return hipGetLastError() == hipSuccess ? 0 : MATGPTQ_GLUE_ELAUNCH; }
+
+}  // namespace
+
+extern "C" {
+
+int matgptq_glue_add_rmsnorm(void* h, const void* delta, const void* weight, void* x, int64_t M, int64_t H,
+                             float eps, void* stream) {
+  if (!h || !weight || !x) return MATGPTQ_GLUE_ENULL;
+  if (M <= 0 || H <= 0 || H % 8 != 0) return MATGPTQ_GLUE_ESHAPE;
+  if (H > 8 * kThreads * kMaxChunks || M > 65535) return MATGPTQ_GLUE_ESIZE;
+  hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)M), dim3(kThreads), 0, (hipStream_t)stream,
+                     (_Float16*)h, (const _Float16*)delta, (const _Float16*)weight, (_Float16*)x, (int)H, eps);
+  return launch_status();
+}
+
+int matgptq_glue_rope_cache(void* qkv, const void* cos_table, const void* sin_table, const int64_t* pos,
+                            void* k_cache, void* v_cache, int64_t M, int heads, int kv_heads, int head_dim,
+                            int64_t max_ctx, void* stream) {
+  if (!qkv || !cos_table || !sin_table || !pos || !k_cache || !v_cache) return MATGPTQ_GLUE_ENULL;
+  if (M <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim <= 0 || head_dim % 2 != 0 ||
+      max_ctx <= 0)
+    return MATGPTQ_GLUE_ESHAPE;
+  if (M > 65535) return MATGPTQ_GLUE_ESIZE;
+  hipLaunchKernelGGL(rope_cache_kernel, dim3((unsigned)(heads + 2 * kv_heads), (unsigned)M), dim3(64), 0,
+                     (hipStream_t)stream, (_Float16*)qkv, (const _Float16*)cos_table, (const _Float16*)sin_table,
+                     pos, (_Float16*)k_cache, (_Float16*)v_cache, heads, kv_heads, head_dim, max_ctx);
+  return launch_status();
+}
+
+int matgptq_glue_attention(const void* qkv, const void* k_cache, const void* v_cache, const int64_t* pos,
+                           void* out, int64_t M, int heads, int kv_heads, int head_dim, int64_t max_ctx,
+                           void* stream) {
+  if (!qkv || !k_cache || !v_cache || !pos || !out) return MATGPTQ_GLUE_ENULL;
+  if (M <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim != 128 || max_ctx <= 0)
+    return MATGPTQ_GLUE_ESHAPE;
+  if (M > 65535 || max_ctx > MATGPTQ_GLUE_MAX_CONTEXT) return MATGPTQ_GLUE_ESIZE;
+  const size_t lds = ((size_t)max_ctx + 16 * 128 + 4) * sizeof(float);
+  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)heads, (unsigned)M), dim3(kThreads), lds,
+                     (hipStream_t)stream, (const _Float16*)qkv, (const _Float16*)k_cache,
+                     (const _Float16*)v_cache, pos, (_Float16*)out, heads, kv_heads, max_ctx,
+                     1.0f / sqrtf((float)head_dim));
+  return launch_status();
+}
+
+int matgptq_glue_silu_mul(const void* gate_up, void* out, int64_t M, int64_t F, void* stream) {
+  if (!gate_up || !out) return MATGPTQ_GLUE_ENULL;
+  if (M <= 0 || F <= 0 || F % 8 != 0) return MATGPTQ_GLUE_ESHAPE;
+  const int64_t blocks = (M * (F / 8) + kThreads - 1) / kThreads;
+  if (blocks > 0x7fffffff) return MATGPTQ_GLUE_ESIZE;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream,
+                     (const _Float16*)gate_up, (_Float16*)out, M, F);
+  return launch_status();
+}
+
+const char* matgptq_glue_strerror(int code) {
+  switch (code) {
+    case 0: return "ok";
+    case MATGPTQ_GLUE_ESHAPE: return "a size is not positive or not divisible as the operator requires";
+    case MATGPTQ_GLUE_ENULL: return "a required pointer is NULL";
+    case MATGPTQ_GLUE_ELAUNCH: return "the HIP runtime reported an error at launch";
+    case MATGPTQ_GLUE_ESIZE: return "a size exceeds what the operator supports";
+    default: return "unknown error";
+  }
+}
+
+}  // extern "C"

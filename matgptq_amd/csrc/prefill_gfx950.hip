@@ -57,14 +57,24 @@ constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && (rbw == 4 || rbw == 2) && mt == 8; }
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
+// LDS of a workgroup, in halves: the ring loop keeps four unpadded buffers of 64 columns, the
+// staged loops two padded ones.
+constexpr int prefill_lds_halves(int rbw, int mt) {
+  return prefill_lean(rbw, mt) ? 4 * 16 * mt * kXs : 2 * 16 * mt * kXsPitch;
+}
+
+// One workgroup tile: activation rows [mtile * 16 MT, +16 MT) x the weight rows of the row blocks
+// rb_base + [nt * 4 RBW, +4 RBW), where lid = nt * m_tiles + mtile.  `lds` is the workgroup's
+// LDS (prefill_lds_halves(RBW, MT) halves, 16-byte aligned).
 template <int BITS, int GROUP, bool ZP, int RBW, int MT>
-__global__ void __launch_bounds__(256, prefill_min_waves(RBW, MT))
-prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
+__device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_tiles, int rb_base,
+                                             _Float16* lds) {
   constexpr int TM = 16 * MT;
   constexpr int GPT = GROUP == 32 ? 4 : 1;
   constexpr int XCHUNKS = TM * (kXs / 8) / 256;  // 16-byte chunks per thread per stage
   static_assert(TM * (kXs / 8) % 256 == 0, "activation tile must split evenly over 256 threads");
-  __shared__ __align__(16) _Float16 xs[2][prefill_lean(RBW, MT) ? 8 : TM * kXsPitch];  // (unused by the ring loop)
+  constexpr int kXsBuf = TM * kXsPitch;  // halves per buffer of the staged loops
+  _Float16* const xs = lds;              // [2][kXsBuf] (unused by the ring loop)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -72,18 +82,10 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   const int r16 = lane & 15;
   const int q = lane >> 4;
 
-  // Tile order.  Workgroup ids go round-robin over the 8 XCDs, each with its own L2.  The
-  // staged tiles remap the ids so that the workgroups of one XCD (ids congruent modulo 8) walk
-  // consecutive activation tiles of the same weight rows; the ring tile measured 2-4 % faster
-  // in the plain order (every 8th activation tile of all weight tiles on one XCD: two
-  // activation tiles, 4 MB, stay in its L2).
-  const int total = n_tiles * m_tiles;
-  int lid = blockIdx.x;
-  if (!prefill_lean(RBW, MT) && (total & 7) == 0) lid = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
   const int nt = lid / m_tiles;
   const int mtile = lid - nt * m_tiles;
   const int m0 = mtile * TM;
-  const int rb_first = (nt * 4 + wave) * RBW;
+  const int rb_first = rb_base + (nt * 4 + wave) * RBW;
 
   constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
   const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
@@ -158,7 +160,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   auto store_x = [&](const u32x4 (&xr)[XCHUNKS], int buf) {
 #pragma unroll
     for (int c = 0; c < XCHUNKS; c++)
-      *reinterpret_cast<half8*>(&xs[buf][x_lds[c]]) = storage8_to_half8(__builtin_bit_cast(half8, xr[c]));
+      *reinterpret_cast<half8*>(&xs[buf * kXsBuf + x_lds[c]]) = storage8_to_half8(__builtin_bit_cast(half8, xr[c]));
   };
 
   auto dequant_step = [&](Frag (&aw)[RBW], const uint32_t (&w)[RBW][BITS], const uint32_t (&s)[RBW][GPT],
@@ -189,7 +191,7 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     }
   };
   auto read_frag = [&](Frag& b, int i, int buf, int jj) {
-    b.v = *reinterpret_cast<const uint4*>(&xs[buf][(i * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
+    b.v = *reinterpret_cast<const uint4*>(&xs[buf * kXsBuf + (i * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
   };
   // One 32-column step of the software pipeline: the matrix cores multiply `aw` by the
   // activation operands `b`; as soon as the MFMAs that use b[i] have been issued, b[i] is
@@ -229,10 +231,10 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     // 16-byte bank groups.  The waits for these copies are written by hand: vmcnt counts every
     // buffer load of the wave in issue order, and each wait below names how many younger ones
     // may still be in flight (see the issue order at the loop).
-    __shared__ __align__(16) _Float16 ring0[TM * kXs];
-    __shared__ __align__(16) _Float16 ring1[TM * kXs];
-    __shared__ __align__(16) _Float16 ring2[TM * kXs];
-    __shared__ __align__(16) _Float16 ring3[TM * kXs];
+    _Float16* const ring0 = lds;
+    _Float16* const ring1 = lds + TM * kXs;
+    _Float16* const ring2 = lds + 2 * TM * kXs;
+    _Float16* const ring3 = lds + 3 * TM * kXs;
     static_assert(TM == 128, "the copy below moves 32 rows per wave");
     // this lane's part of a copy: rows wave*32 + i*8 + lane/8, LDS chunk lane%8
     uint32_t dma_voff[4];
@@ -452,6 +454,54 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   }
 }
 
+template <int BITS, int GROUP, bool ZP, int RBW, int MT>
+__global__ void __launch_bounds__(256, prefill_min_waves(RBW, MT))
+prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
+  __shared__ __align__(16) _Float16 lds[prefill_lds_halves(RBW, MT)];
+  // Tile order.  Workgroup ids go round-robin over the 8 XCDs, each with its own L2.  The
+  // staged tiles remap the ids so that the workgroups of one XCD (ids congruent modulo 8) walk
+  // consecutive activation tiles of the same weight rows; the ring tile measured 2-4 % faster
+  // in the plain order (every 8th activation tile of all weight tiles on one XCD: two
+  // activation tiles, 4 MB, stay in its L2).
+  const int total = n_tiles * m_tiles;
+  int lid = blockIdx.x;
+  if (!prefill_lean(RBW, MT) && (total & 7) == 0) lid = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+  prefill_body<BITS, GROUP, ZP, RBW, MT>(a, lid, m_tiles, 0, lds);
+}
+
+// 128 x 256 tiles with a tail of 128 x 128 tiles.  The larger tile keeps 512 workgroups
+// resident (two per CU); when a layer gives it a whole number of such rounds plus a fraction,
+// that fraction would run as one more round at the full length of a tile.  Here the first
+// `n_big` workgroups take the 128 x 256 tiles of the weight rows below row block `rb_tail`, and
+// the rest of the rows go to workgroups with tiles of half the width, which come last, spread
+// over twice as many CUs and finish in about half the time.
+template <int BITS, int GROUP, bool ZP>
+__global__ void __launch_bounds__(256, 2)
+prefill_tail_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
+  static_assert(prefill_lds_halves(4, 8) == prefill_lds_halves(2, 8), "both tiles share one LDS block");
+  __shared__ __align__(16) _Float16 lds[prefill_lds_halves(4, 8)];
+  if ((int)blockIdx.x < n_big)
+    prefill_body<BITS, GROUP, ZP, 4, 8>(a, blockIdx.x, m_tiles, 0, lds);
+  else
+    prefill_body<BITS, GROUP, ZP, 2, 8>(a, blockIdx.x - n_big, m_tiles, rb_tail, lds);
+}
+
+template <int GROUP, bool ZP>
+hipError_t launch_tail(const GemmArgs& a, hipStream_t stream) {
+  if constexpr (kBf16) {
+    return hipErrorInvalidValue;  // (bf16 storage has no ring loop)
+  } else {
+    const int m_tiles = (a.M + 127) / 128;
+    const int nb = prefill_tail_big_tiles(a.row_blocks, m_tiles);
+    const int rb_tail = nb * 16;
+    const int n_small = (a.row_blocks - rb_tail + 7) / 8;
+    const dim3 grid((nb + n_small) * m_tiles), block(256);
+    hipLaunchKernelGGL((prefill_tail_kernel<kBits, GROUP, ZP>), grid, block, 0, stream, a, m_tiles,
+                       nb * m_tiles, rb_tail);
+    return hipGetLastError();
+  }
+}
+
 template <int GROUP, bool ZP, int RBW, int MT>
 hipError_t launch_cfg(const GemmArgs& a, hipStream_t stream) {
   const int n_tiles = (a.row_blocks + 4 * RBW - 1) / (4 * RBW);
@@ -472,6 +522,7 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 4: return launch_cfg<GROUP, ZP, 2, 2>(a, s);   // 32 x 128
     case 5: return launch_cfg<GROUP, ZP, 8, 4>(a, s);   // 64 x 512
     case 6: return launch_cfg<GROUP, ZP, 8, 2>(a, s);   // 32 x 512
+    case 8: return launch_tail<GROUP, ZP>(a, s);        // 128 x 256, then a tail of 128 x 128
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 }

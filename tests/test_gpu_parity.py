@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(8))
+@pytest.mark.parametrize("cfg", range(9))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -428,3 +428,24 @@ def test_prefill_tiles_agree_bit_for_bit(b, g, zp):
     assert torch.isfinite(staged.float()).all()
     for y in ring:
         assert torch.equal(y, staged)
+
+
+@pytest.mark.parametrize("b,g,zp,n,k,m", [(4, 128, True, 10240, 512, 2048), (3, 32, False, 8192 + 304, 256, 2000),
+                                          (8, -1, True, 4096 + 16, 384, 4096), (2, 128, False, 528, 128, 130)])
+def test_prefill_tail_of_narrow_tiles(b, g, zp, n, k, m):
+    # 128 x 256 tiles for the whole rounds of resident workgroups, 128 x 128 tiles for the rest of
+    # the weight rows, in one launch: same products in the same order as the plain 128 x 256 tile
+    # (first case: the shape split of a Llama-3-70B qkv layer at M = 2048; then ragged N and M, a
+    # tail of a single row block, and a layer with no whole round at all)
+    rng = np.random.default_rng(b)
+    packed = torch.from_numpy(rng.integers(-2 ** 31, 2 ** 31, _lib.load().matgptq_packed_words(b, n, k),
+                                           dtype=np.int64).astype(np.int32)).to(G.DEV)
+    groups = n * (1 if g == -1 else k // g)
+    scales = torch.from_numpy((rng.random(groups) * 0.01 + 1e-3).astype(np.float16)).to(G.DEV)
+    zeros = torch.from_numpy(rng.integers(0, 256, groups).astype(np.float16)).to(G.DEV) if zp else None
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float16)).to(G.DEV)
+    plain = G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (64 << 8)).clone()
+    tail = G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (72 << 8)).clone()
+    torch.cuda.synchronize()
+    assert torch.isfinite(plain.float()).all()
+    assert torch.equal(tail, plain)

@@ -140,3 +140,16 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(8, 128, 4096, 4096, 128, True) == "midbatch b8 g128 zp1 R2 mb2"
     assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).startswith("prefill")
     assert _lib.describe_plan(4, 128, 4096, 4096, 16, True, 1 | (1 << 8)).startswith("decode")
+
+
+def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
+    # 640 tiles of 128 x 256 are one round of 512 resident workgroups and a quarter: the rows of
+    # the quarter go to narrower tiles; whole rounds, or more than half a round left over, keep the
+    # plain tile; bf16 storage has no such kernel
+    assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True).endswith("cfg8")
+    assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 57344, 8192, 2048, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
+    assert not _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3).endswith("cfg8")
+    with pytest.raises(RuntimeError):
+        _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8))
