@@ -1,6 +1,7 @@
 """In-tree build of the native libraries (hipcc cross-compiles gfx950 without a GPU).
 
   libmatgptq_hip.so   the C ABI (include/matgptq_abi.h): HIP kernels + host packers
+  libmatgptq_glue.so  decode-time operators between the linears (include/matgptq_glue.h)
   _C.so               the PyTorch extension that registers the torch ops on top of it
 
 Both land in `matgptq_amd/lib/` so that a source snapshot carries them along.
@@ -19,6 +20,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "lib", "obj")
 ABI_SO = os.path.join(LIBDIR, "libmatgptq_hip.so")
 TORCH_SO = os.path.join(LIBDIR, "_C.so")
+GLUE_SO = os.path.join(LIBDIR, "libmatgptq_glue.so")
 
 BITS = (2, 3, 4, 6, 8)
 ARCH = "gfx950"
@@ -110,8 +112,17 @@ def build_torch_ext(verbose: bool = False) -> str:
     return TORCH_SO
 
 
+def build_glue(verbose: bool = False) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    out = _run([_hipcc(), *HIP_FLAGS, "-shared", os.path.join(CSRC, "glue_gfx950.hip"), "-o", GLUE_SO])
+    if verbose and out.strip():
+        print(out)
+    return GLUE_SO
+
+
 def build_all(verbose: bool = False) -> None:
     build_abi(verbose=verbose)
+    build_glue(verbose=verbose)
     build_torch_ext(verbose=verbose)
 
 

@@ -27,7 +27,7 @@ __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
   return v;
 }
-// sum / maximum over the 256 threads of a workgroup; `red` holds 4 floats and is reused, so the
+// sum over the 256 threads of a workgroup; `red` holds 4 floats and is reused, so the
 // leading barrier keeps a later call from overwriting values an earlier one is still reading
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);
@@ -36,14 +36,6 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   __syncthreads();
   return red[0] + red[1] + red[2] + red[3];
 }
-__device__ __forceinline__ float block_max(float v, float* red) {
-  v = wave_max(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-}
-
 // h += delta (if given); x = h * rsqrt(mean(h^2) + eps) * weight.  One workgroup per row; a thread
 // keeps its chunks of the row in registers (H <= 8 * 256 * kMaxChunks).
 constexpr int kMaxChunks = 4;
@@ -116,18 +108,36 @@ rope_cache_kernel(_Float16* __restrict__ qkv, const _Float16* __restrict__ cos_t
 }
 
 // Attention of one query head of one row over the cache positions 0 .. pos[m] (head dimension
-// 128).  Sixteen lanes share a cache row (16 bytes each), sixteen rows per step of the workgroup;
-// the scores wait in LDS for the softmax, then the same walk accumulates the values.
-// Grid (heads, M), 256 threads, dynamic LDS: max_ctx floats + 16 x 128 floats + 4.
-__global__ void __launch_bounds__(kThreads)
+// 128).  The kernel is bound by the latency of its cache reads, not by their volume, so it runs
+// wide: 1024 threads, sixteen lanes share a cache row (16 bytes each), 64 rows per step of the
+// workgroup and four steps in flight per thread.  The scores wait in LDS for the softmax, then
+// the same walk accumulates the values.
+// Grid (heads, M), dynamic LDS: max_ctx floats + 16 x 128 floats + 16.
+constexpr int kAttnThreads = 1024;
+constexpr int kAttnWaves = kAttnThreads / 64;
+constexpr int kAttnRows = kAttnThreads / 16;  // cache rows per step
+constexpr int kAttnDepth = 4;                 // steps in flight
+
+__device__ __forceinline__ float attn_block_reduce(float v, float* red, bool is_max) {
+  v = is_max ? wave_max(v) : wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = red[0];
+#pragma unroll
+  for (int w = 1; w < kAttnWaves; w++) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+  return r;
+}
+
+__global__ void __launch_bounds__(kAttnThreads)
 attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ k_cache,
                  const _Float16* __restrict__ v_cache, const int64_t* __restrict__ pos,
                  _Float16* __restrict__ out, int heads, int kv_heads, int64_t max_ctx, float scale) {
   extern __shared__ __align__(16) float lds[];
   constexpr int d = 128;
-  float* scores = lds;                 // [max_ctx]
-  float* part = lds + max_ctx;         // [16][128]
-  float* red = part + 16 * d;          // [4]
+  float* scores = lds;                  // [max_ctx]
+  float* part = lds + max_ctx;          // [kAttnWaves][128]
+  float* red = part + kAttnWaves * d;   // [kAttnWaves]
   const int head = blockIdx.x, m = blockIdx.y;
   const int kvh = head / (heads / kv_heads);
   int64_t p = pos[m];
@@ -142,40 +152,68 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
   const _Float16* kb = k_cache + (size_t)kvh * max_ctx * d + sub * 8;
   const _Float16* vb = v_cache + (size_t)kvh * max_ctx * d + sub * 8;
 
+  // (a row beyond n re-reads row n - 1 and is not used: every load is unconditional)
   float mx = -INFINITY;
-  for (int t = grp; t < n; t += 16) {
-    const half8 kv = *reinterpret_cast<const half8*>(kb + (size_t)t * d);
-    float dot = 0.f;
+  for (int t0 = grp; t0 < n; t0 += kAttnRows * kAttnDepth) {
+    half8 kv[kAttnDepth];
 #pragma unroll
-    for (int e = 0; e < 8; e++) dot += q[e] * (float)kv[e];
+    for (int u = 0; u < kAttnDepth; u++) {
+      const int t = t0 + u * kAttnRows;
+      kv[u] = *reinterpret_cast<const half8*>(kb + (size_t)(t < n ? t : n - 1) * d);
+    }
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);  // the 16 lanes of a row are adjacent
-    if (sub == 0) scores[t] = dot;
-    mx = fmaxf(mx, dot);
+    for (int u = 0; u < kAttnDepth; u++) {
+      const int t = t0 + u * kAttnRows;
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) dot += q[e] * (float)kv[u][e];
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);  // the 16 lanes of a row are adjacent
+      if (t < n) {
+        if (sub == 0) scores[t] = dot;
+        mx = fmaxf(mx, dot);
+      }
+    }
   }
-  mx = block_max(mx, red);  // (its barriers also publish the scores)
+  mx = attn_block_reduce(mx, red, true);  // (its barriers also publish the scores)
   float sum = 0.f;
-  for (int t = threadIdx.x; t < n; t += kThreads) {
+  for (int t = threadIdx.x; t < n; t += kAttnThreads) {
     const float e = __expf(scores[t] - mx);
     scores[t] = e;
     sum += e;
   }
-  sum = block_sum(sum, red);
+  sum = attn_block_reduce(sum, red, false);
 
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int t = grp; t < n; t += 16) {
-    const float pr = scores[t];
-    const half8 vv = *reinterpret_cast<const half8*>(vb + (size_t)t * d);
+  for (int t0 = grp; t0 < n; t0 += kAttnRows * kAttnDepth) {
+    half8 vv[kAttnDepth];
+    float pr[kAttnDepth];
 #pragma unroll
-    for (int e = 0; e < 8; e++) acc[e] += pr * (float)vv[e];
+    for (int u = 0; u < kAttnDepth; u++) {
+      const int t = t0 + u * kAttnRows;
+      vv[u] = *reinterpret_cast<const half8*>(vb + (size_t)(t < n ? t : n - 1) * d);
+      pr[u] = t < n ? scores[t] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < kAttnDepth; u++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[e] += pr[u] * (float)vv[u][e];
   }
+  // the four rows of a wave first, then the sixteen waves through LDS
 #pragma unroll
-  for (int e = 0; e < 8; e++) part[grp * d + sub * 8 + e] = acc[e];
+  for (int e = 0; e < 8; e++) {
+    acc[e] += __shfl_xor(acc[e], 16, 64);
+    acc[e] += __shfl_xor(acc[e], 32, 64);
+  }
+  if ((threadIdx.x & 63) < 16) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) part[(threadIdx.x >> 6) * d + sub * 8 + e] = acc[e];
+  }
   __syncthreads();
   if (threadIdx.x < d) {
     float o = 0.f;
 #pragma unroll
-    for (int g = 0; g < 16; g++) o += part[g * d + threadIdx.x];
+    for (int w = 0; w < kAttnWaves; w++) o += part[w * d + threadIdx.x];
     out[((size_t)m * heads + head) * d + threadIdx.x] = (_Float16)(o / sum);
   }
 }
@@ -237,8 +275,8 @@ int matgptq_glue_attention(const void* qkv, const void* k_cache, const void* v_c
   if (M <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim != 128 || max_ctx <= 0)
     return MATGPTQ_GLUE_ESHAPE;
   if (M > 65535 || max_ctx > MATGPTQ_GLUE_MAX_CONTEXT) return MATGPTQ_GLUE_ESIZE;
-  const size_t lds = ((size_t)max_ctx + 16 * 128 + 4) * sizeof(float);
-  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)heads, (unsigned)M), dim3(kThreads), lds,
+  const size_t lds = ((size_t)max_ctx + kAttnWaves * 128 + kAttnWaves) * sizeof(float);
+  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)heads, (unsigned)M), dim3(kAttnThreads), lds,
                      (hipStream_t)stream, (const _Float16*)qkv, (const _Float16*)k_cache,
                      (const _Float16*)v_cache, pos, (_Float16*)out, heads, kv_heads, max_ctx,
                      1.0f / sqrtf((float)head_dim));

@@ -11,8 +11,11 @@ Counterpart of the reference's transformers path:
 
 The reference wraps the step in `torch.compile(mode="reduce-overhead")` to get a device graph;
 here the step is written with device-side position and token tensors and captured directly
-(`torch.cuda.CUDAGraph` is a HIP graph on ROCm).  Only the linears are the product: norms,
-rotary embedding, attention and the head are plain torch operators.
+(`torch.cuda.CUDAGraph` is a HIP graph on ROCm).  The linears are the product.  The operators
+between them are plain torch operators for a prompt, and four small fused HIP kernels
+(`_glue`: residual add + RMS norm, rotary embedding + cache write, attention over the cache,
+SiLU gate) for decode steps of up to 16 rows in fp16, where some twenty separate torch kernels
+per block took twice the time of the linears; the head is a dense torch linear.
 
     python -m matgptq_amd.decoder [--layers 32] [--context 512] [--new_tokens 64] [--bits 2 3 4 6 8]
 """
@@ -124,6 +127,25 @@ class Block(torch.nn.Module):
         h = h + self.down(torch.nn.functional.silu(gu[:, :cfg.ffn]) * gu[:, cfg.ffn:])
         return h
 
+    def forward_fused(self, h, delta, x, cos_table, sin_table, pos, k_cache, v_cache):
+        """The same block for a few rows with the operators between the linears fused (nine
+        launches): `h` [M, hidden] is updated in place with `delta` (the previous block's last
+        linear output, or None) and this block's attention output; returns the output of `down`,
+        which the next block (or the final norm) adds.  `x` [M, hidden] is scratch."""
+        from . import _glue
+
+        cfg = self.cfg
+        m = h.shape[0]
+        _glue.add_rmsnorm(h, delta, self.input_norm, x, cfg.rms_eps)
+        qkv = self.qkv(x)
+        _glue.rope_cache(qkv, cos_table, sin_table, pos, k_cache, v_cache, cfg.heads, cfg.kv_heads)
+        attn = torch.empty(m, cfg.hidden, dtype=h.dtype, device=h.device)
+        _glue.attention(qkv, k_cache, v_cache, pos, attn, cfg.heads, cfg.kv_heads)
+        _glue.add_rmsnorm(h, self.o(attn), self.post_norm, x, cfg.rms_eps)
+        act = torch.empty(m, cfg.ffn, dtype=h.dtype, device=h.device)
+        _glue.silu_mul(self.gate_up(x), act)
+        return self.down(act)
+
 
 def _rotate(t, cos, sin):
     """Rotary embedding, half-split convention: t [M, heads, d], cos/sin [M, d]."""
@@ -149,16 +171,33 @@ class Decoder(torch.nn.Module):
         self.register_buffer("sin", ang.sin().to(embed.dtype).to(embed.device), persistent=False)
         self.register_buffer("arange", torch.arange(max_context, device=embed.device), persistent=False)
         self.max_context = max_context
+        self.fused = True  # decode steps of a few rows use the fused operators between the linears
 
     def new_cache(self):
         cfg = self.cfg
         shape = (len(self.blocks), 2, cfg.kv_heads, self.max_context, cfg.head_dim)
         return torch.zeros(shape, dtype=self.embed.dtype, device=self.embed.device)
 
+    def fused_applies(self, rows: int) -> bool:
+        """The fused operators cover a few fp16 rows at head dimension 128 on a cache they can hold."""
+        from . import _glue
+
+        return (self.fused and rows <= 16 and self.embed.dtype == torch.float16 and self.cfg.head_dim == 128
+                and self.max_context <= _glue.MAX_CONTEXT and self.cfg.hidden <= 8192)
+
     @torch.no_grad()
     def forward(self, tokens, pos, cache):
         """tokens int64 [M], pos int64 [M] (their positions) -> logits [M, vocab] (fp32)."""
         h = self.embed.index_select(0, tokens)
+        if self.fused_applies(h.shape[0]):
+            from . import _glue
+
+            x = torch.empty_like(h)
+            delta = None
+            for i, block in enumerate(self.blocks):
+                delta = block.forward_fused(h, delta, x, self.cos, self.sin, pos, cache[i, 0], cache[i, 1])
+            _glue.add_rmsnorm(h, delta, self.final_norm, x, self.cfg.rms_eps)
+            return torch.nn.functional.linear(x[-1:], self.head).float()
         cos, sin = self.cos.index_select(0, pos), self.sin.index_select(0, pos)
         rep = self.cfg.heads // self.cfg.kv_heads
         bias = torch.where(self.arange[None, :] <= pos[:, None], 0.0, float("-inf")).to(h.dtype).repeat(rep, 1)
