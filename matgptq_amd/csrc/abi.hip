@@ -114,6 +114,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       const int nb = prefill_tail_big_tiles(row_blocks, m_tiles);
       const int64_t rest = (int64_t)((row_blocks - nb * 16 + 15) / 16) * m_tiles;
       if (nb > 0 && rest > 0 && rest <= 256) p->cfg = 8;
+      // Two register sets of 6-bit codes (and of 8-bit codes with zero points) for four row
+      // blocks do not fit beside the accumulators of the 128 x 256 tile: it spills and runs at
+      // half the rate of the 128 x 128 ring tile (8192 x 8192, M = 2048, 6 bits: 596 against
+      // 281 us; 8 bits with zero points: 316 against 269 us).
+      if (bits == 6 || (bits == 8 && zp)) p->cfg = 3;
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
       // (4 bits, Llama-3-8B and 70B layers, M = 17 .. 1024), in microseconds:

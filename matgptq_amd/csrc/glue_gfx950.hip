@@ -110,13 +110,13 @@ rope_cache_kernel(_Float16* __restrict__ qkv, const _Float16* __restrict__ cos_t
 // Attention of one query head of one row over the cache positions 0 .. pos[m] (head dimension
 // 128).  The kernel is bound by the latency of its cache reads, not by their volume, so it runs
 // wide: 1024 threads, sixteen lanes share a cache row (16 bytes each), 64 rows per step of the
-// workgroup and four steps in flight per thread.  The scores wait in LDS for the softmax, then
+// workgroup and eight steps in flight per thread.  The scores wait in LDS for the softmax, then
 // the same walk accumulates the values.
 // Grid (heads, M), dynamic LDS: max_ctx floats + 16 x 128 floats + 16.
 constexpr int kAttnThreads = 1024;
 constexpr int kAttnWaves = kAttnThreads / 64;
 constexpr int kAttnRows = kAttnThreads / 16;  // cache rows per step
-constexpr int kAttnDepth = 4;                 // steps in flight
+constexpr int kAttnDepth = 8;                 // steps in flight
 
 __device__ __forceinline__ float attn_block_reduce(float v, float* red, bool is_max) {
   v = is_max ? wave_max(v) : wave_sum(v);
@@ -153,13 +153,19 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
   const _Float16* vb = v_cache + (size_t)kvh * max_ctx * d + sub * 8;
 
   // (a row beyond n re-reads row n - 1 and is not used: every load is unconditional)
+  auto row_of = [&](int t) { return (size_t)(t < n ? t : n - 1) * d; };
+  // The value rows of the first trip do not depend on the scores: they are requested together
+  // with the key rows, so that a context of up to 64 x kAttnDepth rows costs one round trip to
+  // memory instead of two.
+  half8 v_first[kAttnDepth];
   float mx = -INFINITY;
   for (int t0 = grp; t0 < n; t0 += kAttnRows * kAttnDepth) {
     half8 kv[kAttnDepth];
 #pragma unroll
-    for (int u = 0; u < kAttnDepth; u++) {
-      const int t = t0 + u * kAttnRows;
-      kv[u] = *reinterpret_cast<const half8*>(kb + (size_t)(t < n ? t : n - 1) * d);
+    for (int u = 0; u < kAttnDepth; u++) kv[u] = *reinterpret_cast<const half8*>(kb + row_of(t0 + u * kAttnRows));
+    if (t0 == grp) {
+#pragma unroll
+      for (int u = 0; u < kAttnDepth; u++) v_first[u] = *reinterpret_cast<const half8*>(vb + row_of(t0 + u * kAttnRows));
     }
 #pragma unroll
     for (int u = 0; u < kAttnDepth; u++) {
@@ -191,7 +197,7 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
 #pragma unroll
     for (int u = 0; u < kAttnDepth; u++) {
       const int t = t0 + u * kAttnRows;
-      vv[u] = *reinterpret_cast<const half8*>(vb + (size_t)(t < n ? t : n - 1) * d);
+      vv[u] = t0 == grp ? v_first[u] : *reinterpret_cast<const half8*>(vb + row_of(t));
       pr[u] = t < n ? scores[t] : 0.f;
     }
 #pragma unroll
