@@ -46,8 +46,15 @@ add_rmsnorm_kernel(_Float16* __restrict__ h, const _Float16* __restrict__ delta,
   const int chunks = H / 8;
   half8* hr = reinterpret_cast<half8*>(h + (size_t)blockIdx.x * H);
   const half8* dr = delta ? reinterpret_cast<const half8*>(delta + (size_t)blockIdx.x * H) : nullptr;
-  half8 v[kMaxChunks];
+  const half8* wr = reinterpret_cast<const half8*>(weight);
+  half8 v[kMaxChunks], w[kMaxChunks];
   float ss = 0.f;
+  // (the weights are requested together with the row: one round trip to memory, not two)
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; i++) {
+    const int c = threadIdx.x + i * kThreads;
+    if (c < chunks) w[i] = wr[c];
+  }
 #pragma unroll
   for (int i = 0; i < kMaxChunks; i++) {
     const int c = threadIdx.x + i * kThreads;
@@ -63,15 +70,13 @@ add_rmsnorm_kernel(_Float16* __restrict__ h, const _Float16* __restrict__ delta,
   }
   const float rs = rsqrtf(block_sum(ss, red) / (float)H + eps);
   half8* xr = reinterpret_cast<half8*>(x + (size_t)blockIdx.x * H);
-  const half8* wr = reinterpret_cast<const half8*>(weight);
 #pragma unroll
   for (int i = 0; i < kMaxChunks; i++) {
     const int c = threadIdx.x + i * kThreads;
     if (c < chunks) {
-      const half8 w = wr[c];
       half8 o;
 #pragma unroll
-      for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)v[i][e] * rs * (float)w[e]);
+      for (int e = 0; e < 8; e++) o[e] = (_Float16)((float)v[i][e] * rs * (float)w[i][e]);
       xr[c] = o;
     }
   }
@@ -152,21 +157,16 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
   const _Float16* kb = k_cache + (size_t)kvh * max_ctx * d + sub * 8;
   const _Float16* vb = v_cache + (size_t)kvh * max_ctx * d + sub * 8;
 
-  // (a row beyond n re-reads row n - 1 and is not used: every load is unconditional)
-  auto row_of = [&](int t) { return (size_t)(t < n ? t : n - 1) * d; };
+  // Every load is unconditional and its address does not wait for pos[m]: a row beyond n is
+  // read from inside the cache (beyond the cache: its last row) and never used.
+  const int last = (int)max_ctx - 1;
+  auto row_of = [&](int t) { return (size_t)(t < last ? t : last) * d; };
   // The value rows of the first trip do not depend on the scores: they are requested together
   // with the key rows, so that a context of up to 64 x kAttnDepth rows costs one round trip to
   // memory instead of two.
   half8 v_first[kAttnDepth];
   float mx = -INFINITY;
-  for (int t0 = grp; t0 < n; t0 += kAttnRows * kAttnDepth) {
-    half8 kv[kAttnDepth];
-#pragma unroll
-    for (int u = 0; u < kAttnDepth; u++) kv[u] = *reinterpret_cast<const half8*>(kb + row_of(t0 + u * kAttnRows));
-    if (t0 == grp) {
-#pragma unroll
-      for (int u = 0; u < kAttnDepth; u++) v_first[u] = *reinterpret_cast<const half8*>(vb + row_of(t0 + u * kAttnRows));
-    }
+  auto score_trip = [&](int t0, const half8 (&kv)[kAttnDepth]) {
 #pragma unroll
     for (int u = 0; u < kAttnDepth; u++) {
       const int t = t0 + u * kAttnRows;
@@ -180,6 +180,22 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
         mx = fmaxf(mx, dot);
       }
     }
+  };
+  {
+    // first trip, by every row group whatever n is: nothing here waits for pos[m] before the
+    // loads are on their way
+    half8 kv[kAttnDepth];
+#pragma unroll
+    for (int u = 0; u < kAttnDepth; u++) kv[u] = *reinterpret_cast<const half8*>(kb + row_of(grp + u * kAttnRows));
+#pragma unroll
+    for (int u = 0; u < kAttnDepth; u++) v_first[u] = *reinterpret_cast<const half8*>(vb + row_of(grp + u * kAttnRows));
+    score_trip(grp, kv);
+  }
+  for (int t0 = grp + kAttnRows * kAttnDepth; t0 < n; t0 += kAttnRows * kAttnDepth) {
+    half8 kv[kAttnDepth];
+#pragma unroll
+    for (int u = 0; u < kAttnDepth; u++) kv[u] = *reinterpret_cast<const half8*>(kb + row_of(t0 + u * kAttnRows));
+    score_trip(t0, kv);
   }
   mx = attn_block_reduce(mx, red, true);  // (its barriers also publish the scores)
   float sum = 0.f;
@@ -201,9 +217,12 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
       pr[u] = t < n ? scores[t] : 0.f;
     }
 #pragma unroll
-    for (int u = 0; u < kAttnDepth; u++)
+    for (int u = 0; u < kAttnDepth; u++) {
+      if (t0 + u * kAttnRows < n) {  // (an unused row may hold anything, also NaN)
 #pragma unroll
-      for (int e = 0; e < 8; e++) acc[e] += pr[u] * (float)vv[u][e];
+        for (int e = 0; e < 8; e++) acc[e] += pr[u] * (float)vv[u][e];
+      }
+    }
   }
   // the four rows of a wave first, then the sixteen waves through LDS
 #pragma unroll

@@ -78,7 +78,11 @@ def test_attention(m, heads, kv, ctx, positions):
     v_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
     pos = torch.tensor(positions, device=DEV)
     out = torch.full((m, heads * d), float("nan"), device=DEV, dtype=torch.float16)
-    _glue.attention(qkv, k_cache, v_cache, pos, out, heads, kv)
+    # rows no query may see hold NaN for the kernel (it reads some of them, and must not use them)
+    k_dirty, v_dirty = k_cache.clone(), v_cache.clone()
+    k_dirty[:, max(positions) + 1:] = float("nan")
+    v_dirty[:, max(positions) + 1:] = float("nan")
+    _glue.attention(qkv, k_dirty, v_dirty, pos, out, heads, kv)
     q = qkv.view(m, heads + 2 * kv, d)[:, :heads].float()
     rep = heads // kv
     k = k_cache.float().repeat_interleave(rep, dim=0)  # [heads, ctx, d]
