@@ -355,14 +355,16 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
 
   auto run_stages = [&](int c0, int c1, int n_stages) {
     if constexpr (STREAM) {
-      // two stages per trip so that the prefetched stage needs no register copy
+      // two stages per trip so that the prefetched stage needs no register copy.  Every trip
+      // issues both loads whether or not those stages exist (a stage past the end reads through
+      // zero-length descriptors): with a branch around a load the compiler has to assume the
+      // fewer loads in flight of the two paths, and its wait before the current stage's first
+      // use would then also wait for the stage just requested.
       for (int stage = 0; stage < n_stages; stage += 2) {
-        if (stage + 1 < n_stages) load_stage(nxt, c0, c1, stage + 1);
+        load_stage(nxt, c0, c1, stage + 1);
         compute_stage(cur, c0, c1, stage);
-        if (stage + 1 < n_stages) {
-          if (stage + 2 < n_stages) load_stage(cur, c0, c1, stage + 2);
-          compute_stage(nxt, c0, c1, stage + 1);
-        }
+        load_stage(cur, c0, c1, stage + 2);
+        compute_stage(nxt, c0, c1, stage + 1);
       }
     } else {
       for (int stage = 0; stage < n_stages; stage++) {
