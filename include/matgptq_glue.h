@@ -51,6 +51,14 @@ int matgptq_glue_attention(const void *qkv, const void *k_cache, const void *v_c
                            const int64_t *pos, void *out, int64_t M, int heads, int kv_heads,
                            int head_dim, int64_t max_ctx, void *stream);
 
+/* matgptq_glue_rope_cache followed by matgptq_glue_attention for a single row (M = 1) in one
+ * launch, with the same results: qkv is read only (the rotated query stays in registers),
+ * k_cache and v_cache receive row pos[0], out[1, heads * head_dim] the attention output. */
+int matgptq_glue_rope_attention(const void *qkv, const void *cos_table, const void *sin_table,
+                                const int64_t *pos, void *k_cache, void *v_cache, void *out,
+                                int heads, int kv_heads, int head_dim, int64_t max_ctx,
+                                void *stream);
+
 /* out[M,F] = silu(gate_up[M, 0:F]) * gate_up[M, F:2F].  F % 8 == 0. */
 int matgptq_glue_silu_mul(const void *gate_up, void *out, int64_t M, int64_t F, void *stream);
 

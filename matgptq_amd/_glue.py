@@ -17,7 +17,7 @@ GLUE_PATH = os.path.join(_HERE, "lib", "libmatgptq_glue.so")
 MAX_CONTEXT = 8192
 
 EXPORTS = ("matgptq_glue_strerror", "matgptq_glue_add_rmsnorm", "matgptq_glue_rope_cache",
-           "matgptq_glue_attention", "matgptq_glue_silu_mul")
+           "matgptq_glue_attention", "matgptq_glue_rope_attention", "matgptq_glue_silu_mul")
 
 _lib = None
 
@@ -40,6 +40,7 @@ def load() -> ctypes.CDLL:
     L.matgptq_glue_add_rmsnorm.argtypes = [vp, vp, vp, vp, i64, i64, f32, vp]
     L.matgptq_glue_rope_cache.argtypes = [vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, i64, vp]
     L.matgptq_glue_attention.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, i64, vp]
+    L.matgptq_glue_rope_attention.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, i64, vp]
     L.matgptq_glue_silu_mul.argtypes = [vp, vp, i64, i64, vp]
     for name in EXPORTS[1:]:
         getattr(L, name).restype = ci
@@ -103,6 +104,20 @@ def attention(qkv, k_cache, v_cache, pos, out, heads: int, kv_heads: int) -> Non
         raise GlueError("attention: shapes differ")
     _check(load().matgptq_glue_attention(qkv.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), pos.data_ptr(),
                                          out.data_ptr(), m, heads, kv_heads, d, max_ctx, _stream()))
+
+
+def rope_attention(qkv, cos, sin, pos, k_cache, v_cache, out, heads: int, kv_heads: int) -> None:
+    """`rope_cache` and `attention` for one row in one launch (same results; qkv is left as it is)."""
+    _f16(qkv, cos, sin, k_cache, v_cache, out)
+    _pos_ok(pos, 1)
+    kv, max_ctx, d = k_cache.shape
+    if (qkv.shape[0] != 1 or kv != kv_heads or v_cache.shape != k_cache.shape
+            or qkv.shape[1] != (heads + 2 * kv_heads) * d or cos.shape != (max_ctx, d) or sin.shape != (max_ctx, d)
+            or out.shape != (1, heads * d)):
+        raise GlueError("rope_attention: shapes differ")
+    _check(load().matgptq_glue_rope_attention(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), pos.data_ptr(),
+                                              k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), heads,
+                                              kv_heads, d, max_ctx, _stream()))
 
 
 def silu_mul(gate_up, out) -> None:

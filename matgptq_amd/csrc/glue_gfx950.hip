@@ -82,6 +82,13 @@ add_rmsnorm_kernel(_Float16* __restrict__ h, const _Float16* __restrict__ delta,
   }
 }
 
+// One element of the rotary embedding: own * cos + other * sin, where `other` is the partner of
+// the half-split pair with its sign (minus the upper partner for the lower half, plus the lower
+// partner for the upper half).  One expression for every kernel, so that all of them round alike.
+__device__ __forceinline__ _Float16 rotary(float own, float other, _Float16 c, _Float16 s) {
+  return (_Float16)(own * (float)c + other * (float)s);
+}
+
 // Rotary embedding (half-split pairs) of the query and key heads of one row of the fused qkv
 // output; queries are rotated in place, rotated keys and the values go to row pos[m] of the
 // caches [kv_heads, max_ctx, d].  Grid (heads + 2 kv_heads, M), 64 threads.
@@ -105,10 +112,8 @@ rope_cache_kernel(_Float16* __restrict__ qkv, const _Float16* __restrict__ cos_t
   const int half = d / 2;
   for (int i = threadIdx.x; i < half; i += 64) {
     const float a = (float)src[i], b = (float)src[i + half];
-    const float lo = a * (float)c[i] - b * (float)s[i];
-    const float hi = b * (float)c[i + half] + a * (float)s[i + half];
-    dst[i] = (_Float16)lo;
-    dst[i + half] = (_Float16)hi;
+    dst[i] = rotary(a, -b, c[i], s[i]);
+    dst[i + half] = rotary(b, a, c[i + half], s[i + half]);
   }
 }
 
@@ -134,10 +139,17 @@ __device__ __forceinline__ float attn_block_reduce(float v, float* red, bool is_
   return r;
 }
 
+// ROPE (one query row only): the rotary embedding and the cache write of the row happen here as
+// well, which saves a launch per block.  The query head is rotated in registers; the row's own
+// key (rotated) and value come from qkv instead of the cache, and the workgroup of the first
+// query head of each key/value head writes them to the caches for the steps to come (another
+// workgroup may read that cache row meanwhile: it does not use what it read).
+template <bool ROPE>
 __global__ void __launch_bounds__(kAttnThreads)
-attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ k_cache,
-                 const _Float16* __restrict__ v_cache, const int64_t* __restrict__ pos,
-                 _Float16* __restrict__ out, int heads, int kv_heads, int64_t max_ctx, float scale) {
+attention_kernel(const _Float16* __restrict__ qkv, _Float16* k_cache, _Float16* v_cache,
+                 const int64_t* __restrict__ pos, _Float16* __restrict__ out,
+                 const _Float16* __restrict__ cos_t, const _Float16* __restrict__ sin_t, int heads,
+                 int kv_heads, int64_t max_ctx, float scale) {
   extern __shared__ __align__(16) float lds[];
   constexpr int d = 128;
   float* scores = lds;                  // [max_ctx]
@@ -150,10 +162,13 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
   const int n = (int)p + 1;
   const int sub = threadIdx.x & 15, grp = threadIdx.x >> 4;
 
-  const half8 qv = *reinterpret_cast<const half8*>(qkv + ((size_t)m * (heads + 2 * kv_heads) + head) * d + sub * 8);
-  float q[8];
-#pragma unroll
-  for (int e = 0; e < 8; e++) q[e] = (float)qv[e] * scale;
+  const _Float16* row = qkv + (size_t)m * (heads + 2 * kv_heads) * d + sub * 8;
+  half8 qv = *reinterpret_cast<const half8*>(row + (size_t)head * d);
+  half8 k_cur = qv, v_cur = qv;
+  if constexpr (ROPE) {
+    k_cur = *reinterpret_cast<const half8*>(row + (size_t)(heads + kvh) * d);
+    v_cur = *reinterpret_cast<const half8*>(row + (size_t)(heads + kv_heads + kvh) * d);
+  }
   const _Float16* kb = k_cache + (size_t)kvh * max_ctx * d + sub * 8;
   const _Float16* vb = v_cache + (size_t)kvh * max_ctx * d + sub * 8;
 
@@ -164,15 +179,39 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
   // The value rows of the first trip do not depend on the scores: they are requested together
   // with the key rows, so that a context of up to 64 x kAttnDepth rows costs one round trip to
   // memory instead of two.
-  half8 v_first[kAttnDepth];
+  half8 v_first[kAttnDepth], k_first[kAttnDepth];
+#pragma unroll
+  for (int u = 0; u < kAttnDepth; u++) k_first[u] = *reinterpret_cast<const half8*>(kb + row_of(grp + u * kAttnRows));
+#pragma unroll
+  for (int u = 0; u < kAttnDepth; u++) v_first[u] = *reinterpret_cast<const half8*>(vb + row_of(grp + u * kAttnRows));
+  if constexpr (ROPE) {
+    // lanes sub and sub ^ 8 of a row group hold the two halves of the rotary pairs
+    const half8 cv = *reinterpret_cast<const half8*>(cos_t + (size_t)p * d + sub * 8);
+    const half8 sv = *reinterpret_cast<const half8*>(sin_t + (size_t)p * d + sub * 8);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float qo = (float)qv[e], ko = (float)k_cur[e];
+      const float qp = __shfl_xor(qo, 8, 64), kp = __shfl_xor(ko, 8, 64);
+      qv[e] = rotary(qo, sub < 8 ? -qp : qp, cv[e], sv[e]);
+      k_cur[e] = rotary(ko, sub < 8 ? -kp : kp, cv[e], sv[e]);
+    }
+    if (head % (heads / kv_heads) == 0 && grp == 0) {
+      *reinterpret_cast<half8*>(k_cache + ((size_t)kvh * max_ctx + p) * d + sub * 8) = k_cur;
+      *reinterpret_cast<half8*>(v_cache + ((size_t)kvh * max_ctx + p) * d + sub * 8) = v_cur;
+    }
+  }
+  float q[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) q[e] = (float)qv[e] * scale;
   float mx = -INFINITY;
   auto score_trip = [&](int t0, const half8 (&kv)[kAttnDepth]) {
 #pragma unroll
     for (int u = 0; u < kAttnDepth; u++) {
       const int t = t0 + u * kAttnRows;
+      const half8 kk = ROPE && t == (int)p ? k_cur : kv[u];
       float dot = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; e++) dot += q[e] * (float)kv[u][e];
+      for (int e = 0; e < 8; e++) dot += q[e] * (float)kk[e];
 #pragma unroll
       for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);  // the 16 lanes of a row are adjacent
       if (t < n) {
@@ -181,16 +220,9 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
       }
     }
   };
-  {
-    // first trip, by every row group whatever n is: nothing here waits for pos[m] before the
-    // loads are on their way
-    half8 kv[kAttnDepth];
-#pragma unroll
-    for (int u = 0; u < kAttnDepth; u++) kv[u] = *reinterpret_cast<const half8*>(kb + row_of(grp + u * kAttnRows));
-#pragma unroll
-    for (int u = 0; u < kAttnDepth; u++) v_first[u] = *reinterpret_cast<const half8*>(vb + row_of(grp + u * kAttnRows));
-    score_trip(grp, kv);
-  }
+  // first trip, by every row group whatever n is (its rows were requested above, before
+  // anything waited for pos[m])
+  score_trip(grp, k_first);
   for (int t0 = grp + kAttnRows * kAttnDepth; t0 < n; t0 += kAttnRows * kAttnDepth) {
     half8 kv[kAttnDepth];
 #pragma unroll
@@ -214,6 +246,7 @@ attention_kernel(const _Float16* __restrict__ qkv, const _Float16* __restrict__ 
     for (int u = 0; u < kAttnDepth; u++) {
       const int t = t0 + u * kAttnRows;
       vv[u] = t0 == grp ? v_first[u] : *reinterpret_cast<const half8*>(vb + row_of(t));
+      if (ROPE && t == (int)p) vv[u] = v_cur;
       pr[u] = t < n ? scores[t] : 0.f;
     }
 #pragma unroll
@@ -301,10 +334,25 @@ int matgptq_glue_attention(const void* qkv, const void* k_cache, const void* v_c
     return MATGPTQ_GLUE_ESHAPE;
   if (M > 65535 || max_ctx > MATGPTQ_GLUE_MAX_CONTEXT) return MATGPTQ_GLUE_ESIZE;
   const size_t lds = ((size_t)max_ctx + kAttnWaves * 128 + kAttnWaves) * sizeof(float);
-  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)heads, (unsigned)M), dim3(kAttnThreads), lds,
-                     (hipStream_t)stream, (const _Float16*)qkv, (const _Float16*)k_cache,
-                     (const _Float16*)v_cache, pos, (_Float16*)out, heads, kv_heads, max_ctx,
-                     1.0f / sqrtf((float)head_dim));
+  hipLaunchKernelGGL(attention_kernel<false>, dim3((unsigned)heads, (unsigned)M), dim3(kAttnThreads), lds,
+                     (hipStream_t)stream, (const _Float16*)qkv, (_Float16*)k_cache, (_Float16*)v_cache, pos,
+                     (_Float16*)out, (const _Float16*)nullptr, (const _Float16*)nullptr, heads, kv_heads,
+                     max_ctx, 1.0f / sqrtf((float)head_dim));
+  return launch_status();
+}
+
+int matgptq_glue_rope_attention(const void* qkv, const void* cos_table, const void* sin_table,
+                                const int64_t* pos, void* k_cache, void* v_cache, void* out, int heads,
+                                int kv_heads, int head_dim, int64_t max_ctx, void* stream) {
+  if (!qkv || !cos_table || !sin_table || !pos || !k_cache || !v_cache || !out) return MATGPTQ_GLUE_ENULL;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim != 128 || max_ctx <= 0)
+    return MATGPTQ_GLUE_ESHAPE;
+  if (max_ctx > MATGPTQ_GLUE_MAX_CONTEXT) return MATGPTQ_GLUE_ESIZE;
+  const size_t lds = ((size_t)max_ctx + kAttnWaves * 128 + kAttnWaves) * sizeof(float);
+  hipLaunchKernelGGL(attention_kernel<true>, dim3((unsigned)heads, 1u), dim3(kAttnThreads), lds,
+                     (hipStream_t)stream, (const _Float16*)qkv, (_Float16*)k_cache, (_Float16*)v_cache, pos,
+                     (_Float16*)out, (const _Float16*)cos_table, (const _Float16*)sin_table, heads, kv_heads,
+                     max_ctx, 1.0f / sqrtf((float)head_dim));
   return launch_status();
 }
 

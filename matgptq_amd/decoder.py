@@ -131,16 +131,20 @@ class Block(torch.nn.Module):
         """The same block for a few rows with the operators between the linears fused (nine
         launches): `h` [M, hidden] is updated in place with `delta` (the previous block's last
         linear output, or None) and this block's attention output; returns the output of `down`,
-        which the next block (or the final norm) adds.  `x` [M, hidden] is scratch."""
+        which the next block (or the final norm) adds.  `x` [M, hidden] is scratch.  Eight launches
+        for a single row."""
         from . import _glue
 
         cfg = self.cfg
         m = h.shape[0]
         _glue.add_rmsnorm(h, delta, self.input_norm, x, cfg.rms_eps)
         qkv = self.qkv(x)
-        _glue.rope_cache(qkv, cos_table, sin_table, pos, k_cache, v_cache, cfg.heads, cfg.kv_heads)
         attn = torch.empty(m, cfg.hidden, dtype=h.dtype, device=h.device)
-        _glue.attention(qkv, k_cache, v_cache, pos, attn, cfg.heads, cfg.kv_heads)
+        if m == 1:  # rotary embedding, cache write and attention in one launch
+            _glue.rope_attention(qkv, cos_table, sin_table, pos, k_cache, v_cache, attn, cfg.heads, cfg.kv_heads)
+        else:
+            _glue.rope_cache(qkv, cos_table, sin_table, pos, k_cache, v_cache, cfg.heads, cfg.kv_heads)
+            _glue.attention(qkv, k_cache, v_cache, pos, attn, cfg.heads, cfg.kv_heads)
         _glue.add_rmsnorm(h, self.o(attn), self.post_norm, x, cfg.rms_eps)
         act = torch.empty(m, cfg.ffn, dtype=h.dtype, device=h.device)
         _glue.silu_mul(self.gate_up(x), act)

@@ -94,6 +94,35 @@ def test_attention(m, heads, kv, ctx, positions):
     assert err <= 2e-3 * max(1.0, float(ref.abs().max()))  # fp32 throughout, one fp16 rounding of the result
 
 
+@pytest.mark.parametrize("heads,kv,ctx,position", [(32, 8, 600, 511), (4, 2, 64, 0), (8, 8, 1000, 999), (4, 1, 300, 64)])
+def test_rope_attention_equals_the_two_launches(heads, kv, ctx, position):
+    from matgptq_amd import _glue
+
+    d = 128
+    g = _gen(ctx + heads)
+    qkv = torch.randn(1, (heads + 2 * kv) * d, device=DEV, generator=g).half()
+    ang = torch.rand(ctx, d, device=DEV, generator=g) * 6.28
+    cos, sin = ang.cos().half(), ang.sin().half()
+    pos = torch.tensor([position], device=DEV)
+    k_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
+    v_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
+    k_cache[:, position + 1:] = float("nan")
+    v_cache[:, position + 1:] = float("nan")
+    qkv_two, k_two, v_two = qkv.clone(), k_cache.clone(), v_cache.clone()
+    out_two = torch.empty(1, heads * d, device=DEV, dtype=torch.float16)
+    _glue.rope_cache(qkv_two, cos, sin, pos, k_two, v_two, heads, kv)
+    _glue.attention(qkv_two, k_two, v_two, pos, out_two, heads, kv)
+    qkv_one, k_one, v_one = qkv.clone(), k_cache.clone(), v_cache.clone()
+    out_one = torch.full((1, heads * d), float("nan"), device=DEV, dtype=torch.float16)
+    _glue.rope_attention(qkv_one, cos, sin, pos, k_one, v_one, out_one, heads, kv)
+    # same arithmetic in the same order: the same bits
+    assert torch.equal(out_one, out_two)
+    assert torch.equal(k_one[:, :position + 1], k_two[:, :position + 1])
+    assert torch.equal(v_one[:, :position + 1], v_two[:, :position + 1])
+    assert torch.equal(qkv_one, qkv)  # read only
+    assert torch.isnan(k_one[:, position + 1:]).all() and torch.isnan(v_one[:, position + 1:]).all()
+
+
 @pytest.mark.parametrize("m,f", [(1, 14336), (7, 512), (16, 1000)])
 def test_silu_mul(m, f):
     from matgptq_amd import _glue
