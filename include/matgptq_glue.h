@@ -59,6 +59,21 @@ int matgptq_glue_rope_attention(const void *qkv, const void *cos_table, const vo
                                 int heads, int kv_heads, int head_dim, int64_t max_ctx,
                                 void *stream);
 
+/* The same attention with the context split over workgroups (one per key/value head and 64
+ * cache rows, serving all query heads of that key/value head) and a second small launch that
+ * combines their partial results: for short batches, where a workgroup per query head leaves
+ * most of the GPU idle.  Query heads per key/value head: 1, 2, 4 or 8.  fuse_rotary != 0 (M = 1
+ * only) also does what matgptq_glue_rope_cache does, like matgptq_glue_rope_attention;
+ * otherwise qkv holds rotated queries and the caches are read only (cos_table / sin_table may
+ * be NULL).  workspace: matgptq_glue_attention_workspace_floats() floats, contents irrelevant
+ * before and after; calls that share a workspace must not overlap.  Results agree with
+ * matgptq_glue_attention to the fp32 rounding of the softmax sums. */
+size_t matgptq_glue_attention_workspace_floats(int64_t M, int heads, int64_t max_ctx);
+int matgptq_glue_attention_split(const void *qkv, const void *cos_table, const void *sin_table,
+                                 const int64_t *pos, void *k_cache, void *v_cache, void *out,
+                                 void *workspace, int64_t M, int heads, int kv_heads,
+                                 int head_dim, int64_t max_ctx, int fuse_rotary, void *stream);
+
 /* out[M,F] = silu(gate_up[M, 0:F]) * gate_up[M, F:2F].  F % 8 == 0. */
 int matgptq_glue_silu_mul(const void *gate_up, void *out, int64_t M, int64_t F, void *stream);
 

@@ -17,7 +17,8 @@ GLUE_PATH = os.path.join(_HERE, "lib", "libmatgptq_glue.so")
 MAX_CONTEXT = 8192
 
 EXPORTS = ("matgptq_glue_strerror", "matgptq_glue_add_rmsnorm", "matgptq_glue_rope_cache",
-           "matgptq_glue_attention", "matgptq_glue_rope_attention", "matgptq_glue_silu_mul")
+           "matgptq_glue_attention", "matgptq_glue_rope_attention", "matgptq_glue_attention_workspace_floats",
+           "matgptq_glue_attention_split", "matgptq_glue_silu_mul")
 
 _lib = None
 
@@ -42,8 +43,11 @@ def load() -> ctypes.CDLL:
     L.matgptq_glue_attention.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, i64, vp]
     L.matgptq_glue_rope_attention.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, i64, vp]
     L.matgptq_glue_silu_mul.argtypes = [vp, vp, i64, i64, vp]
+    L.matgptq_glue_attention_split.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, i64, ci, vp]
+    L.matgptq_glue_attention_workspace_floats.argtypes = [i64, ci, i64]
     for name in EXPORTS[1:]:
         getattr(L, name).restype = ci
+    L.matgptq_glue_attention_workspace_floats.restype = ctypes.c_size_t
     _lib = L
     return L
 
@@ -118,6 +122,33 @@ def rope_attention(qkv, cos, sin, pos, k_cache, v_cache, out, heads: int, kv_hea
     _check(load().matgptq_glue_rope_attention(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), pos.data_ptr(),
                                               k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), heads,
                                               kv_heads, d, max_ctx, _stream()))
+
+
+def attention_workspace(rows: int, heads: int, max_ctx: int, device):
+    """Workspace of `attention_split` for up to `rows` query rows (contents irrelevant)."""
+    floats = load().matgptq_glue_attention_workspace_floats(rows, heads, max_ctx)
+    return torch.empty(floats, dtype=torch.float32, device=device)
+
+
+def attention_split(qkv, cos, sin, pos, k_cache, v_cache, out, workspace, heads: int, kv_heads: int,
+                    fuse_rotary: bool) -> None:
+    """`attention` with the context split over workgroups; with `fuse_rotary` (one row) also the
+    rotary embedding and the cache write, like `rope_attention`."""
+    _f16(qkv, k_cache, v_cache, out, *((cos, sin) if fuse_rotary else ()))
+    m = qkv.shape[0]
+    _pos_ok(pos, m)
+    kv, max_ctx, d = k_cache.shape
+    if (kv != kv_heads or v_cache.shape != k_cache.shape or qkv.shape[1] != (heads + 2 * kv_heads) * d
+            or out.shape != (m, heads * d) or (fuse_rotary and (cos.shape != (max_ctx, d) or sin.shape != (max_ctx, d)))):
+        raise GlueError("attention_split: shapes differ")
+    need = load().matgptq_glue_attention_workspace_floats(m, heads, max_ctx)
+    if (workspace.dtype != torch.float32 or not workspace.is_cuda or not workspace.is_contiguous()
+            or workspace.numel() < need):
+        raise GlueError("attention_split: workspace too small or of the wrong type")
+    _check(load().matgptq_glue_attention_split(
+        qkv.data_ptr(), cos.data_ptr() if fuse_rotary else None, sin.data_ptr() if fuse_rotary else None,
+        pos.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), workspace.data_ptr(),
+        m, heads, kv_heads, d, max_ctx, int(fuse_rotary), _stream()))
 
 
 def silu_mul(gate_up, out) -> None:

@@ -17,6 +17,8 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
 constexpr int kThreads = 256;
 
+int launch_status() { return hipGetLastError() == hipSuccess ? 0 : MATGPTQ_GLUE_ELAUNCH; }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -276,6 +278,211 @@ attention_kernel(const _Float16* __restrict__ qkv, _Float16* k_cache, _Float16* 
   }
 }
 
+// The same attention with the context split over workgroups: grid (kv_heads, splits, M), one
+// workgroup per key/value head and 64 cache rows, which serves all REP query heads of that
+// key/value head from one read of the rows (a workgroup per query head reads them REP times, and
+// a single CU can pull only so much).  Every workgroup with rows to look at leaves its partial
+// result - the maximum score, the sum of the exponentials and the weighted values, per query
+// head - in `ws`; attention_combine_kernel, launched behind it, puts the partial results of the
+// splits up to pos[m] together.  (One kernel whose last workgroup combines was measured slower:
+// the fences that publish the partial results across the L2 caches of the XCDs cost more than
+// the second launch.)
+// ws: M x heads x splits x 130 floats.
+constexpr int kSplitRows = 64;
+constexpr int kSplitStride = 130;  // 128 values, maximum, sum
+
+template <bool ROPE, int REP>
+__global__ void __launch_bounds__(256)
+attention_split_kernel(const _Float16* __restrict__ qkv, _Float16* k_cache, _Float16* v_cache,
+                       const int64_t* __restrict__ pos, _Float16* __restrict__ out,
+                       const _Float16* __restrict__ cos_t, const _Float16* __restrict__ sin_t,
+                       float* __restrict__ ws, int heads, int kv_heads, int64_t max_ctx, int splits, float scale) {
+  constexpr int d = 128;
+  __shared__ float sc[REP][kSplitRows];  // scores, then exponentials
+  __shared__ float part[4][REP][d];      // weighted values per wave
+  __shared__ float mx_s[REP], sum_s[REP];
+  const int kvh = blockIdx.x, split = blockIdx.y, m = blockIdx.z;
+  const int tid = threadIdx.x, sub = tid & 15, grp = tid >> 4, wave = tid >> 6, lane = tid & 63;
+  const int row0 = split * kSplitRows;
+  const int last = (int)max_ctx - 1;
+  auto row_of = [&](int t) { return (size_t)(t < last ? t : last) * d; };
+  const _Float16* kb = k_cache + (size_t)kvh * max_ctx * d + sub * 8;
+  const _Float16* vb = v_cache + (size_t)kvh * max_ctx * d + sub * 8;
+  // this thread's rows: row0 + grp + 16 u; requested before anything waits for pos[m]
+  half8 kr[4], vr[4];
+#pragma unroll
+  for (int u = 0; u < 4; u++) kr[u] = *reinterpret_cast<const half8*>(kb + row_of(row0 + grp + 16 * u));
+#pragma unroll
+  for (int u = 0; u < 4; u++) vr[u] = *reinterpret_cast<const half8*>(vb + row_of(row0 + grp + 16 * u));
+  const _Float16* row = qkv + (size_t)m * (heads + 2 * kv_heads) * d + sub * 8;
+  half8 qv[REP];
+#pragma unroll
+  for (int r = 0; r < REP; r++) qv[r] = *reinterpret_cast<const half8*>(row + (size_t)(kvh * REP + r) * d);
+  half8 k_cur = qv[0], v_cur = qv[0];
+  if constexpr (ROPE) {
+    k_cur = *reinterpret_cast<const half8*>(row + (size_t)(heads + kvh) * d);
+    v_cur = *reinterpret_cast<const half8*>(row + (size_t)(heads + kv_heads + kvh) * d);
+  }
+  int64_t p = pos[m];
+  p = p < 0 ? 0 : (p >= max_ctx ? max_ctx - 1 : p);
+  const int n = (int)p + 1;
+  if (row0 >= n) return;  // nothing to look at: the combining kernel skips this split as well
+  if constexpr (ROPE) {
+    const half8 cv = *reinterpret_cast<const half8*>(cos_t + (size_t)p * d + sub * 8);
+    const half8 sv = *reinterpret_cast<const half8*>(sin_t + (size_t)p * d + sub * 8);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float ko = (float)k_cur[e];
+      const float kp = __shfl_xor(ko, 8, 64);
+      k_cur[e] = rotary(ko, sub < 8 ? -kp : kp, cv[e], sv[e]);
+#pragma unroll
+      for (int r = 0; r < REP; r++) {
+        const float qo = (float)qv[r][e];
+        const float qp = __shfl_xor(qo, 8, 64);
+        qv[r][e] = rotary(qo, sub < 8 ? -qp : qp, cv[e], sv[e]);
+      }
+    }
+    // the workgroup whose rows include the new one writes it to the caches
+    if ((int)p >= row0 && (int)p < row0 + kSplitRows && grp == 0) {
+      *reinterpret_cast<half8*>(k_cache + ((size_t)kvh * max_ctx + p) * d + sub * 8) = k_cur;
+      *reinterpret_cast<half8*>(v_cache + ((size_t)kvh * max_ctx + p) * d + sub * 8) = v_cur;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int t = row0 + grp + 16 * u;
+    const half8 kk = ROPE && t == (int)p ? k_cur : kr[u];
+#pragma unroll
+    for (int r = 0; r < REP; r++) {
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) dot += (float)qv[r][e] * scale * (float)kk[e];
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64);
+      if (sub == 0) sc[r][grp + 16 * u] = t < n ? dot : -INFINITY;
+    }
+  }
+  __syncthreads();
+  // maximum and sum of exponentials per query head: wave w takes heads w, w + 4; lane = row
+  for (int r = wave; r < REP; r += 4) {
+    const float v = sc[r][lane];
+    const float mx = wave_max(v);
+    const float e = mx == -INFINITY ? 0.f : __expf(v - mx);
+    sc[r][lane] = e;
+    const float sum = wave_sum(e);
+    if (lane == 0) { mx_s[r] = mx; sum_s[r] = sum; }
+  }
+  __syncthreads();
+  float acc[REP][8];
+#pragma unroll
+  for (int r = 0; r < REP; r++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[r][e] = 0.f;
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int t = row0 + grp + 16 * u;
+    if (t < n) {  // (an unused row may hold anything, also NaN)
+      const half8 vv = ROPE && t == (int)p ? v_cur : vr[u];
+#pragma unroll
+      for (int r = 0; r < REP; r++) {
+        const float pr = sc[r][grp + 16 * u];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[r][e] += pr * (float)vv[e];
+      }
+    }
+  }
+  // the four row groups of a wave by shuffles, the four waves through LDS
+#pragma unroll
+  for (int r = 0; r < REP; r++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      acc[r][e] += __shfl_xor(acc[r][e], 16, 64);
+      acc[r][e] += __shfl_xor(acc[r][e], 32, 64);
+    }
+  if (lane < 16) {
+#pragma unroll
+    for (int r = 0; r < REP; r++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) part[wave][r][sub * 8 + e] = acc[r][e];
+  }
+  __syncthreads();
+  const int head0 = kvh * REP;
+  for (int idx = tid; idx < REP * d; idx += 256) {
+    const int r = idx >> 7, dim = idx & 127;
+    float* dst = ws + ((size_t)(m * heads + head0 + r) * splits + split) * kSplitStride;
+    dst[dim] = part[0][r][dim] + part[1][r][dim] + part[2][r][dim] + part[3][r][dim];
+    if (dim == 0) { dst[128] = mx_s[r]; dst[129] = sum_s[r]; }
+  }
+}
+
+// out[m, head, :] = sum over the splits with rows (those below pos[m] + 1) of the partial values,
+// each weighted by exp(its maximum - the overall maximum), over the sum of the partial sums
+// weighted alike.  Grid (heads, M), 128 threads (one per element of the head).
+__global__ void __launch_bounds__(128)
+attention_combine_kernel(const float* __restrict__ ws, const int64_t* __restrict__ pos, _Float16* __restrict__ out,
+                         int heads, int64_t max_ctx, int splits) {
+  constexpr int d = 128;
+  const int head = blockIdx.x, m = blockIdx.y, dim = threadIdx.x;
+  int64_t p = pos[m];
+  p = p < 0 ? 0 : (p >= max_ctx ? max_ctx - 1 : p);
+  const int used = ((int)p + kSplitRows) / kSplitRows;  // splits that hold rows 0 .. p
+  const float* src = ws + (size_t)(m * heads + head) * splits * kSplitStride;
+  // eight splits at a time, all their loads in flight together (a split beyond the used ones
+  // re-reads the last used one with weight zero); running maximum, sum and value are rescaled
+  // whenever a chunk raises the maximum
+  float mx = -INFINITY, sum = 0.f, o = 0.f;
+  for (int sp0 = 0; sp0 < used; sp0 += 8) {
+    float ms[8], ls[8], vs[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const float* part = src + (size_t)(sp0 + i < used ? sp0 + i : used - 1) * kSplitStride;
+      ms[i] = part[128];
+      ls[i] = part[129];
+      vs[i] = part[dim];
+    }
+    float cm = mx;
+#pragma unroll
+    for (int i = 0; i < 8; i++) cm = fmaxf(cm, ms[i]);
+    const float keep = mx == -INFINITY ? 0.f : __expf(mx - cm);
+    sum *= keep;
+    o *= keep;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const float w = sp0 + i < used ? __expf(ms[i] - cm) : 0.f;
+      sum += w * ls[i];
+      o += w * vs[i];
+    }
+    mx = cm;
+  }
+  out[((size_t)m * heads + head) * d + dim] = (_Float16)(o / sum);
+}
+
+template <bool ROPE>
+int launch_attention_split(const void* qkv, void* k_cache, void* v_cache, const int64_t* pos, void* out,
+                           const void* cos_table, const void* sin_table, void* ws, int64_t M, int heads,
+                           int kv_heads, int64_t max_ctx, void* stream) {
+  const int splits = (int)((max_ctx + kSplitRows - 1) / kSplitRows);
+  const dim3 grid((unsigned)kv_heads, (unsigned)splits, (unsigned)M), block(256);
+  const float scale = 1.0f / sqrtf(128.0f);
+#define MATGPTQ_GLUE_SPLIT(REP)                                                                              \
+  hipLaunchKernelGGL((attention_split_kernel<ROPE, REP>), grid, block, 0, (hipStream_t)stream,                \
+                     (const _Float16*)qkv, (_Float16*)k_cache, (_Float16*)v_cache, pos, (_Float16*)out,       \
+                     (const _Float16*)cos_table, (const _Float16*)sin_table, (float*)ws, heads, kv_heads,   \
+                     max_ctx, splits, scale)
+  switch (heads / kv_heads) {
+    case 1: MATGPTQ_GLUE_SPLIT(1); break;
+    case 2: MATGPTQ_GLUE_SPLIT(2); break;
+    case 4: MATGPTQ_GLUE_SPLIT(4); break;
+    case 8: MATGPTQ_GLUE_SPLIT(8); break;
+    default: return MATGPTQ_GLUE_ESHAPE;
+  }
+#undef MATGPTQ_GLUE_SPLIT
+  if (int e = launch_status()) return e;
+  hipLaunchKernelGGL(attention_combine_kernel, dim3((unsigned)heads, (unsigned)M), dim3(128), 0,
+                     (hipStream_t)stream, (const float*)ws, pos, (_Float16*)out, heads, max_ctx, splits);
+  return launch_status();
+}
+
 // out[m, j] = silu(gu[m, j]) * gu[m, F + j]; both factors rounded to fp16 like the two
 // element-wise operators it replaces.
 __global__ void __launch_bounds__(kThreads)
@@ -295,8 +502,6 @@ silu_mul_kernel(const _Float16* __restrict__ gu, _Float16* __restrict__ out, int
   }
   *reinterpret_cast<half8*>(out + m * F + j * 8) = o;
 }
-
-int launch_status() { return hipGetLastError() == hipSuccess ? 0 : MATGPTQ_GLUE_ELAUNCH; }
 
 }  // namespace
 
@@ -354,6 +559,27 @@ int matgptq_glue_rope_attention(const void* qkv, const void* cos_table, const vo
                      (_Float16*)out, (const _Float16*)cos_table, (const _Float16*)sin_table, heads, kv_heads,
                      max_ctx, 1.0f / sqrtf((float)head_dim));
   return launch_status();
+}
+
+size_t matgptq_glue_attention_workspace_floats(int64_t M, int heads, int64_t max_ctx) {
+  if (M <= 0 || heads <= 0 || max_ctx <= 0) return 0;
+  return (size_t)M * heads * ((max_ctx + kSplitRows - 1) / kSplitRows) * kSplitStride;
+}
+
+int matgptq_glue_attention_split(const void* qkv, const void* cos_table, const void* sin_table,
+                                 const int64_t* pos, void* k_cache, void* v_cache, void* out, void* workspace,
+                                 int64_t M, int heads, int kv_heads, int head_dim, int64_t max_ctx,
+                                 int fuse_rotary, void* stream) {
+  if (!qkv || !pos || !k_cache || !v_cache || !out || !workspace) return MATGPTQ_GLUE_ENULL;
+  if (fuse_rotary && (!cos_table || !sin_table)) return MATGPTQ_GLUE_ENULL;
+  if (M <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || head_dim != 128 || max_ctx <= 0 ||
+      (fuse_rotary && M != 1))
+    return MATGPTQ_GLUE_ESHAPE;
+  if (M > 65535 || max_ctx > MATGPTQ_GLUE_MAX_CONTEXT) return MATGPTQ_GLUE_ESIZE;
+  return fuse_rotary ? launch_attention_split<true>(qkv, k_cache, v_cache, pos, out, cos_table, sin_table,
+                                                    workspace, M, heads, kv_heads, max_ctx, stream)
+                     : launch_attention_split<false>(qkv, k_cache, v_cache, pos, out, cos_table, sin_table,
+                                                     workspace, M, heads, kv_heads, max_ctx, stream);
 }
 
 int matgptq_glue_silu_mul(const void* gate_up, void* out, int64_t M, int64_t F, void* stream) {

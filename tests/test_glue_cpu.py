@@ -33,6 +33,11 @@ def test_argument_checks_come_before_any_launch():
     assert L.matgptq_glue_attention(one, one, one, one, one, 1, 4, 2, 128, _glue.MAX_CONTEXT + 1, None) == -8
     assert L.matgptq_glue_rope_attention(one, one, one, one, one, one, None, 4, 2, 128, 64, None) == -4
     assert L.matgptq_glue_rope_attention(one, one, one, one, one, one, one, 4, 2, 64, 64, None) == -3
+    assert L.matgptq_glue_attention_split(one, None, None, one, one, one, one, None, 1, 4, 2, 128, 64, 0, None) == -4
+    assert L.matgptq_glue_attention_split(one, None, None, one, one, one, one, one, 1, 4, 2, 128, 64, 1, None) == -4
+    assert L.matgptq_glue_attention_split(one, one, one, one, one, one, one, one, 2, 4, 2, 128, 64, 1, None) == -3
+    assert L.matgptq_glue_attention_split(one, None, None, one, one, one, one, one, 1, 6, 2, 128, 64, 0, None) == -3
+    assert L.matgptq_glue_attention_workspace_floats(2, 4, 65) == 2 * 4 * 2 * 130
     assert L.matgptq_glue_silu_mul(one, None, 1, 64, None) == -4
     assert L.matgptq_glue_silu_mul(one, one, 1, 60, None) == -3
     assert b"NULL" in L.matgptq_glue_strerror(-4)

@@ -123,6 +123,62 @@ def test_rope_attention_equals_the_two_launches(heads, kv, ctx, position):
     assert torch.isnan(k_one[:, position + 1:]).all() and torch.isnan(v_one[:, position + 1:]).all()
 
 
+@pytest.mark.parametrize("m,heads,kv,ctx,positions", [(1, 32, 8, 600, [511]), (3, 4, 2, 64, [0, 17, 63]),
+                                                      (2, 8, 8, 8192, [8191, 300]), (16, 8, 1, 100, list(range(16))),
+                                                      (1, 4, 2, 65, [64]), (2, 2, 1, 130, [5, 129])])
+def test_attention_split_agrees_with_the_unsplit_kernel(m, heads, kv, ctx, positions):
+    from matgptq_amd import _glue
+
+    d = 128
+    g = _gen(ctx + m + heads)
+    qkv = torch.randn(m, (heads + 2 * kv) * d, device=DEV, generator=g).half()
+    k_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
+    v_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
+    k_cache[:, max(positions) + 1:] = float("nan")
+    v_cache[:, max(positions) + 1:] = float("nan")
+    pos = torch.tensor(positions, device=DEV)
+    ref = torch.empty(m, heads * d, device=DEV, dtype=torch.float16)
+    _glue.attention(qkv, k_cache, v_cache, pos, ref, heads, kv)
+    ws = _glue.attention_workspace(m, heads, ctx, DEV)
+    for _ in range(2):
+        ws.fill_(float("nan"))  # nothing may be read from the workspace that this call did not write
+        out = torch.full((m, heads * d), float("nan"), device=DEV, dtype=torch.float16)
+        _glue.attention_split(qkv, None, None, pos, k_cache, v_cache, out, ws, heads, kv, fuse_rotary=False)
+        # fp32 sums in another order, one fp16 rounding of the result
+        assert float((out.float() - ref.float()).abs().max()) <= 2e-3 * max(1.0, float(ref.float().abs().max()))
+
+
+@pytest.mark.parametrize("heads,kv,ctx,position", [(32, 8, 600, 511), (4, 2, 64, 0), (8, 8, 1000, 999), (8, 1, 300, 64),
+                                                   (4, 2, 200, 127), (4, 2, 200, 128)])
+def test_attention_split_with_rotary_equals_the_two_launches(heads, kv, ctx, position):
+    from matgptq_amd import _glue
+
+    d = 128
+    g = _gen(ctx + heads)
+    qkv = torch.randn(1, (heads + 2 * kv) * d, device=DEV, generator=g).half()
+    ang = torch.rand(ctx, d, device=DEV, generator=g) * 6.28
+    cos, sin = ang.cos().half(), ang.sin().half()
+    pos = torch.tensor([position], device=DEV)
+    k_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
+    v_cache = torch.randn(kv, ctx, d, device=DEV, generator=g).half()
+    k_cache[:, position + 1:] = float("nan")
+    v_cache[:, position + 1:] = float("nan")
+    qkv_two, k_two, v_two = qkv.clone(), k_cache.clone(), v_cache.clone()
+    out_two = torch.empty(1, heads * d, device=DEV, dtype=torch.float16)
+    _glue.rope_cache(qkv_two, cos, sin, pos, k_two, v_two, heads, kv)
+    _glue.attention(qkv_two, k_two, v_two, pos, out_two, heads, kv)
+    qkv_one, k_one, v_one = qkv.clone(), k_cache.clone(), v_cache.clone()
+    out_one = torch.full((1, heads * d), float("nan"), device=DEV, dtype=torch.float16)
+    ws = _glue.attention_workspace(1, heads, ctx, DEV).fill_(float("nan"))
+    _glue.attention_split(qkv_one, cos, sin, pos, k_one, v_one, out_one, ws, heads, kv, fuse_rotary=True)
+    assert float((out_one.float() - out_two.float()).abs().max()) <= 2e-3 * max(1.0, float(out_two.float().abs().max()))
+    # the cache rows are the same bits: one rotary expression in every kernel
+    assert torch.equal(k_one[:, :position + 1], k_two[:, :position + 1])
+    assert torch.equal(v_one[:, :position + 1], v_two[:, :position + 1])
+    assert torch.equal(qkv_one, qkv)
+    assert torch.isnan(k_one[:, position + 1:]).all() and torch.isnan(v_one[:, position + 1:]).all()
+
+
 @pytest.mark.parametrize("m,f", [(1, 14336), (7, 512), (16, 1000)])
 def test_silu_mul(m, f):
     from matgptq_amd import _glue
@@ -155,10 +211,12 @@ def _decoder(context=80, seed=5):
     return D, cfg, dec
 
 
+@pytest.mark.parametrize("context", (80, 1100))  # short cache: one attention launch; long: split over workgroups
 @pytest.mark.parametrize("rows", (1, 3))
-def test_fused_step_matches_step_of_torch_operators(rows):
-    D, cfg, dec = _decoder()
+def test_fused_step_matches_step_of_torch_operators(rows, context):
+    D, cfg, dec = _decoder(context)
     assert dec.fused_applies(rows) and not dec.fused_applies(17)
+    assert dec.split_attention == (context > 768)
     prompt = torch.randint(0, cfg.vocab, (30,), device=DEV, generator=_gen(1))
     cache = dec.new_cache()
     dec(prompt, torch.arange(30, device=DEV), cache)  # 30 rows: torch operators
