@@ -118,7 +118,16 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // blocks do not fit beside the accumulators of the 128 x 256 tile: it spills and runs at
       // half the rate of the 128 x 128 ring tile (8192 x 8192, M = 2048, 6 bits: 596 against
       // 281 us; 8 bits with zero points: 316 against 269 us).
-      if (bits == 6 || (bits == 8 && zp)) p->cfg = 3;
+      // Between the two, a 128 x 192 tile (three row blocks per wave) fits the registers and runs
+      // about 9 % faster per weight than the 128 x 128 tile where its tiles fill the rounds of 512
+      // resident workgroups as well (57344 x 8192, 6 bits: 1748 against 1906 us; on 8192 rows, 43
+      // tiles of 192, it only ties).  Rounds times tile width decide.
+      if (bits == 6 || (bits == 8 && zp)) {
+        const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
+        const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
+        const double t_128 = (double)((wgs_128 + 511) / 512);
+        p->cfg = t_192 < t_128 ? 9 : 3;
+      }
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
       // (4 bits, Llama-3-8B and 70B layers, M = 17 .. 1024), in microseconds:
@@ -172,7 +181,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       R = 1 << ((variant - 80) % 3);
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
-      if (variant - 64 > 8) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 9) return MATGPTQ_EVARIANT;
       if (variant - 64 == 8 && (flags & MATGPTQ_FLAG_BF16)) return MATGPTQ_EVARIANT;  // ring loop: fp16 storage only
       p->decode = false;
       p->skinny = false;

@@ -54,7 +54,7 @@ constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 // that budget runs the ring loop below (activations straight into LDS, one operand set).
 // (bf16 storage: the copy into LDS would bypass the bf16 -> fp16 conversion, so that build keeps
 // the staged loop for this tile as well)
-constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && (rbw == 4 || rbw == 2) && mt == 8; }
+constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && (rbw == 4 || rbw == 3 || rbw == 2) && mt == 8; }
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
 // LDS of a workgroup, in halves: the ring loop keeps four unpadded buffers of 64 columns, the
@@ -294,16 +294,18 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
           acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, bv[i].h, acc[rr][i], 0, 0, 0);
         ring_frag(bv[i], nring, i, njj);
       }
-      constexpr int kHalf = (RBW / 2) * MT;           // MFMAs per half
-      constexpr int kValuHalf = (RBW / 2) * 26;       // vector instructions of two row blocks, roughly
+      constexpr int kHalf = (RBW / 2) * MT;              // MFMAs of the first half
+      constexpr int kRest = (RBW - RBW / 2) * MT;        // ... of the second (one more row block when RBW is odd)
+      constexpr int kValuHalf = (RBW / 2) * 26;          // vector instructions of the first half's row blocks, roughly
+      constexpr int kValuRest = (RBW - RBW / 2) * 26;
       __builtin_amdgcn_sched_group_barrier(0x002, kValuHalf, 0);
 #pragma unroll
       for (int n = 0; n < kHalf; n++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, (kValuHalf + kHalf - 1) / kHalf, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (kValuRest + kHalf - 1) / kHalf, 0);
       }
 #pragma unroll
-      for (int n = 0; n < kHalf; n++) {
+      for (int n = 0; n < kRest; n++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if (n & 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
@@ -523,6 +525,7 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 5: return launch_cfg<GROUP, ZP, 8, 4>(a, s);   // 64 x 512
     case 6: return launch_cfg<GROUP, ZP, 8, 2>(a, s);   // 32 x 512
     case 8: return launch_tail<GROUP, ZP>(a, s);        // 128 x 256, then a tail of 128 x 128
+    case 9: return launch_cfg<GROUP, ZP, 3, 8>(a, s);   // 128 x 192
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 }

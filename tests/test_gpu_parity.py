@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(9))
+@pytest.mark.parametrize("cfg", range(10))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -423,6 +423,7 @@ def test_prefill_tiles_agree_bit_for_bit(b, g, zp):
     x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float16)).to(G.DEV)
     ring = [G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (64 << 8)).clone() for _ in range(3)]
     ring.append(G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (67 << 8)).clone())  # 128 x 128 ring tile
+    ring.append(G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (73 << 8)).clone())  # 128 x 192 ring tile
     staged = G.gemm(b, g, n, k, x, packed, scales, zeros, flags=1 | (66 << 8))  # 64 x 256, staged
     torch.cuda.synchronize()
     assert torch.isfinite(staged.float()).all()
