@@ -269,6 +269,22 @@ def test_llama3_70b_layer_prefill_full_size():
     assert np.max(np.abs(y1.astype(np.float64) - y[5:6])) <= 2e-3 * np.max(np.abs(y1.astype(np.float64)))
 
 
+def test_llama3_70b_qkv_prefill_full_size_with_tail_tiles():
+    # 10240 rows at M = 2048: the planner splits the launch into 128 x 256 tiles (rows below 8192)
+    # and a tail of 128 x 128 tiles; rows of both parts against the oracle
+    n, k, m = 10240, 8192, 2048
+    assert _lib.describe_plan(4, 128, n, k, m, True).endswith("cfg8")
+    lay = G.Layer(n, k, 4, 128, seed=0)
+    x = o.make_activations(m, k, seed=0)
+    y = lay.run(x)
+    assert np.all(np.isfinite(y))
+    rows = np.array([0, 130, 1023, 2047])
+    G.assert_close_to_oracle(y[rows], x[rows], lay.w, "70B qkv prefill")
+    tail = y[rows][:, 8192:].astype(np.float64)
+    ref = o.linear_f64(x[rows], lay.w[8192:])
+    assert np.max(np.abs(tail - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+
+
 def test_sync_flag_and_error_paths_on_device():
     lay = G.Layer(32, 256, 4, 128, seed=1)
     x = o.make_activations(2, 256, seed=1)
