@@ -437,6 +437,45 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
 
   }  // pipelined loop
 
+  if constexpr (prefill_lean(RBW, MT) && (RBW == 4 || RBW == 2)) {
+    // Epilogue of the ring tiles through LDS, so that the output leaves in whole row segments: a
+    // lane holds 4 consecutive output columns of one batch row per accumulator (8 bytes, 32 per
+    // row and store), while all workgroups of a round write their tiles at the same time and
+    // the memory system takes 16-byte pieces of full 128-byte (64-byte) row segments better.
+    // The ring is free once every wave is past its last operand read and every copy into it
+    // has landed (also the copies of half tiles beyond K, which write zeros).  A wave owns the
+    // 128 x 16 RBW block of its row blocks: 16-byte chunk c of row r sits at chunk c ^ (r % CH).
+    constexpr int CH = RBW * 2;        // 16-byte chunks per row of the block
+    constexpr int ROWH = RBW * 16;     // halves per row
+    __builtin_amdgcn_s_waitcnt(0);     // vmcnt(0) expcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    _Float16* blk = lds + wave * (TM * ROWH);
+#pragma unroll
+    for (int rr = 0; rr < RBW; rr++) {
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int r = mt * 16 + r16;
+        const int c = rr * 2 + (q >> 1);
+        uint16_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = float_to_storage(acc[rr][mt][i]);
+        *reinterpret_cast<uint2*>(blk + r * ROWH + ((c ^ (r & (CH - 1))) * 8) + (q & 1) * 4) =
+            make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+      }
+    }
+    constexpr int RPI = 64 / CH;  // rows per store instruction
+    const int c = lane % CH;
+    const int rb = rb_first + (c >> 1);
+#pragma unroll
+    for (int i = 0; i < TM / RPI; i++) {
+      const int r = i * RPI + lane / CH;
+      const int m = m0 + r;
+      const uint4 v = *reinterpret_cast<const uint4*>(blk + r * ROWH + ((c ^ (r & (CH - 1))) * 8));
+      if (m < a.M && rb < a.row_blocks)
+        *reinterpret_cast<uint4*>(a.y + (size_t)m * a.N + (size_t)rb_first * 16 + c * 8) = v;
+    }
+    return;
+  }
   // epilogue: lane holds rows (weight rows) 4q..4q+3 of column (batch row) r16
 #pragma unroll
   for (int rr = 0; rr < RBW; rr++) {
