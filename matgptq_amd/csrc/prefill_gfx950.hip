@@ -437,7 +437,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
 
   }  // pipelined loop
 
-  if constexpr (prefill_lean(RBW, MT) && (RBW == 4 || RBW == 2)) {
+  if constexpr (prefill_lean(RBW, MT)) {
     // Epilogue of the ring tiles through LDS, so that the output leaves in whole row segments: a
     // lane holds 4 consecutive output columns of one batch row per accumulator (8 bytes, 32 per
     // row and store), while all workgroups of a round write their tiles at the same time and
@@ -445,8 +445,9 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     // The ring is free once every wave is past its last operand read and every copy into it
     // has landed (also the copies of half tiles beyond K, which write zeros).  A wave owns the
     // 128 x 16 RBW block of its row blocks: 16-byte chunk c of row r sits at chunk c ^ (r % CH).
-    constexpr int CH = RBW * 2;        // 16-byte chunks per row of the block
-    constexpr int ROWH = RBW * 16;     // halves per row
+    // (three row blocks: rows of eight chunks as well, the last two unused)
+    constexpr int CH = RBW == 3 ? 8 : RBW * 2;  // 16-byte chunks per row of the block
+    constexpr int ROWH = CH * 8;                // halves per row
     __builtin_amdgcn_s_waitcnt(0);     // vmcnt(0) expcnt(0) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     _Float16* blk = lds + wave * (TM * ROWH);
@@ -471,7 +472,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       const int r = i * RPI + lane / CH;
       const int m = m0 + r;
       const uint4 v = *reinterpret_cast<const uint4*>(blk + r * ROWH + ((c ^ (r & (CH - 1))) * 8));
-      if (m < a.M && rb < a.row_blocks)
+      if (m < a.M && rb < a.row_blocks && c < RBW * 2)
         *reinterpret_cast<uint4*>(a.y + (size_t)m * a.N + (size_t)rb_first * 16 + c * 8) = v;
     }
     return;
