@@ -52,7 +52,7 @@ def _abi_jobs():
     jobs = []
     # the GEMM kernels are built once per bitwidth and storage type (fp16, bf16); the
     # longest compilations go first so that the pool finishes evenly
-    for stem in ("prefill_gfx950", "decode_gfx950", "skinny_gfx950"):
+    for stem in ("prefill_gfx950", "decode_gfx950", "skinny_gfx950", "gemv_gfx950"):
         for bf16 in (0, 1):
             for b in BITS:
                 obj = os.path.join(OBJDIR, f"{stem}_b{b}{'_bf16' if bf16 else ''}.o")

@@ -19,6 +19,8 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
                                 bool stream_flavour, size_t smem, hipStream_t);                \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);          \
   hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, hipStream_t);   \
+  hipError_t launch_gemv_b##B(const GemmArgs&, int shape, int W, size_t lds_pad, hipStream_t);  \
+  hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int shape, int W, size_t lds_pad, hipStream_t); \
   hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, hipStream_t); \
   hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
                                        int kc, bool stream_flavour, size_t smem, hipStream_t); \
@@ -40,9 +42,16 @@ hipError_t launch_dequant(int, int, int64_t, int64_t, const uint32_t*, const uin
 namespace {
 
 constexpr int kDecodeMaxM = 16;
+constexpr int kGemvMaxM = 4;
+// (tiles per wave and round, row blocks per workgroup) of the gemv kernel's instantiations
+constexpr int kNumGemvShapes = 6;
+constexpr int kGemvShapes[kNumGemvShapes][2] = {{8, 1}, {4, 1}, {4, 2}, {2, 2}, {2, 4}, {2, 1}};
 constexpr size_t kLdsBudget = 64 * 1024;  // dynamic LDS a decode workgroup may ask for
 
 struct Plan {
+  bool gemv;     // batch 1..4 at group 128: gemv kernel, `shape` = its (T, R) entry, W waves
+  int shape;
+  size_t pad;    // gemv: dynamic LDS to ask for at least (bounds the workgroups per CU)
   bool decode;
   bool skinny;   // mid-batch kernel (K split inside the workgroup), R row blocks per workgroup
   int mb;        // mid-batch: blocks of 16 batch rows per workgroup
@@ -75,6 +84,9 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   const int variant = (int)((flags & MATGPTQ_FLAG_VARIANT_MASK) >> MATGPTQ_FLAG_VARIANT_SHIFT);
   const int flavour = (int)((flags >> 16) & 3u);
   p->decode = M <= kDecodeMaxM;
+  p->gemv = false;
+  p->shape = 0;
+  p->pad = 0;
   p->skinny = false;
   p->mb = 2;
   p->cfg = 0;
@@ -173,7 +185,40 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     p->mb = 1;
     R = mid_rows(1);
   }
+  // Batch rows 1..4 at group size 128: the gemv kernel (every wave requests a whole round of
+  // tiles at once).  Measured on MI355X (Llama-3-8B layers, every bitwidth): four tiles per
+  // wave and round; one row block per workgroup at batch 1 and on layers with few row blocks,
+  // two above that (the staged activations of several batch rows are then shared); as many
+  // waves as there are rounds of four tiles, sixteen at most.
+  if (M <= kGemvMaxM && group_size == 128 && flavour == 0 && (variant == 0 || variant >= 100)) {
+    int shape = (M >= 2 && row_blocks >= 320) ? 2 : 1;
+    if (variant >= 100) {
+      shape = variant - 100;
+      if (shape >= kNumGemvShapes) return MATGPTQ_EVARIANT;
+    }
+    const int T = kGemvShapes[shape][0];
+    int Wg = (int)((flags >> MATGPTQ_FLAG_GEMV_WAVES_SHIFT) & 31u);
+    if (Wg == 0) {
+      Wg = (k_tiles + T - 1) / T;
+      if (Wg > 16) Wg = 16;
+    }
+    if (Wg > 16) return MATGPTQ_EVARIANT;
+    p->gemv = true;
+    p->decode = false;
+    p->skinny = false;
+    p->shape = shape;
+    p->R = kGemvShapes[shape][1];
+    p->S = 0;
+    p->W = Wg;
+    p->kc = 0;
+    p->stream = false;
+    p->smem = 0;
+    p->pad = (size_t)((flags >> MATGPTQ_FLAG_GEMV_LDS_SHIFT) & 63u) * 4096u;
+    if (p->pad > 160 * 1024) return MATGPTQ_EVARIANT;
+    return MATGPTQ_OK;
+  }
   if (variant != 0) {
+    if (variant >= 100) return MATGPTQ_EVARIANT;
     if (variant >= 80) {
       if (variant - 80 > 8) return MATGPTQ_EVARIANT;
       p->decode = false;
@@ -262,6 +307,19 @@ hipError_t launch_prefill(int bits, bool bf16, const GemmArgs& a, int g, const P
 #undef MATGPTQ_CASE
 }
 
+hipError_t launch_gemv(int bits, bool bf16, const GemmArgs& a, const Plan& p, hipStream_t s) {
+#define MATGPTQ_CASE(B) \
+  case B: return bf16 ? launch_gemv_b##B##_bf16(a, p.shape, p.W, p.pad, s) : launch_gemv_b##B(a, p.shape, p.W, p.pad, s);
+  switch (bits) {
+    MATGPTQ_CASE(2)
+    MATGPTQ_CASE(3)
+    MATGPTQ_CASE(4)
+    MATGPTQ_CASE(6)
+    default: return bf16 ? launch_gemv_b8_bf16(a, p.shape, p.W, p.pad, s) : launch_gemv_b8(a, p.shape, p.W, p.pad, s);
+  }
+#undef MATGPTQ_CASE
+}
+
 hipError_t launch_skinny(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
 #define MATGPTQ_CASE(B) \
   case B: return bf16 ? launch_skinny_b##B##_bf16(a, g, p.R, p.mb, s) : launch_skinny_b##B(a, g, p.R, p.mb, s);
@@ -323,7 +381,8 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
   a.row_blocks = (int)(N / 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
-  const hipError_t err = p.decode   ? launch_decode(bitwidth, bf16, a, group_size, p, s)
+  const hipError_t err = p.gemv     ? launch_gemv(bitwidth, bf16, a, p, s)
+                         : p.decode ? launch_decode(bitwidth, bf16, a, group_size, p, s)
                          : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, s)
                                     : launch_prefill(bitwidth, bf16, a, group_size, p, s);
   if (err != hipSuccess) return MATGPTQ_ELAUNCH;
@@ -340,7 +399,10 @@ int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, in
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, has_zeros != 0, flags, &p)) return e;
-  if (p.decode)
+  if (p.gemv)
+    snprintf(buf, buf_len, "gemv b%d g%d zp%d T%d R%d W%d pad%zu", bitwidth, group_size, has_zeros ? 1 : 0,
+             kGemvShapes[p.shape][0], p.R, p.W, p.pad);
+  else if (p.decode)
     snprintf(buf, buf_len, "decode-%s b%d g%d zp%d R%d S%d W%d kc%d lds%zu",
              p.kc < (int)(K / 128) ? "chunked" : (p.stream ? "stream" : "burst"), bitwidth, group_size,
              has_zeros ? 1 : 0, p.R, p.S, p.W, p.kc, p.smem);

@@ -1,0 +1,285 @@
+// Batch-1..4 kernel for group size 128: the HBM-bound end of the decode regime.
+// Compiled once per bitwidth with -DMATGPTQ_BITS=b.
+// Role of the reference's gptq_matryoshka_simt
+// (inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:636-953); the design is its own.
+//
+// Work split.  A workgroup of W waves owns R row blocks (16 weight rows each) and all of
+// K.  Wave w owns the tiles [(round W + w) T, +T) of those row blocks, round = 0, 1, ...:
+// T consecutive 128-column tiles, i.e. T contiguous KiB-sized pieces of every row block.
+// A wave requests everything a round needs at once - the activations of its columns, the
+// scales and zeros of its groups, then all R T tiles of codes - and consumes the tiles in
+// request order, so the whole round is in flight while the first tile is multiplied.  The
+// footprint per wave is small (R T b registers of codes) and many waves are resident.
+//
+// Arithmetic.  The vector ALU only masks codes into "raw" fp16 pairs 1024 + c 2^p; the
+// products run on the matrix cores with the ACTIVATIONS as the 16-row operand and the 16
+// weight rows as the 16 columns:  D[i][n] = sum_k A[i][k] raw[n][k].  Row 4u + v of A holds
+// batch row v (scaled by 2^-p, as X') during tile u of a group of four tiles and zeros
+// otherwise, so that one chain of sixteen MFMAs leaves the sums of four tiles side by side:
+// lane (n, q) ends with  sum_k raw X'  of tile q, weight row n, batch rows 0..3 in its four
+// accumulator registers.  The same lane holds the scale and zero of exactly that tile and
+// row (one 2-byte load per lane fetches the scales of four tiles x 16 rows) and the two
+// row-independent sums of that tile,  off = 1024 sum X'  and  xs = sum X, which the wave
+// forms while it stages X' (dot products plus a rotate-reduce over the 16 lanes of a tile):
+//     acc += scale * (D - off - zero / 2^(8-b) * xs)
+// which is  sum_k scale ((c << (8-b)) - zero) x / 2^(8-b)  over the group.  The partial sums
+// of the four lane quarters and the W waves meet in LDS once, at the end.
+#include "device_common.h"
+
+#ifndef MATGPTQ_BITS
+#error "compile with -DMATGPTQ_BITS={2,3,4,6,8}"
+#endif
+
+namespace matgptq {
+
+namespace {
+
+constexpr int kBits = MATGPTQ_BITS;
+
+__device__ __forceinline__ float dot2(half2v a, half2v b, float c) {
+  return __builtin_amdgcn_fdot2(a, b, c, false);
+}
+
+// v + (v rotated right by N lanes inside each row of 16 lanes)
+template <int N>
+__device__ __forceinline__ float add_row_ror(float v) {
+  const int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + N, 0xF, 0xF, false);
+  return v + __int_as_float(r);
+}
+__device__ __forceinline__ float row_sum16(float v) {
+  v = add_row_ror<8>(v);
+  v = add_row_ror<4>(v);
+  v = add_row_ror<2>(v);
+  return add_row_ror<1>(v);
+}
+
+// LDS bytes per wave: X' of one round for MB batch rows + a block of zeros
+constexpr int gemv_wave_lds(int t, int mb) { return mb * t * 256 + 256; }
+
+template <int BITS, bool ZP, int T, int R, int MB>
+__device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
+  constexpr int TH = (T + 3) / 4;  // groups of four tiles per round
+  constexpr float kMul = (float)(1 << (8 - BITS));
+  constexpr int kXBytes = MB * T * 256;
+  constexpr int kWaveBytes = gemv_wave_lds(T, MB);
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15;  // weight row inside the row block / row of the activation operand
+  const int q = lane >> 4;
+  const int rb0 = blockIdx.x * R;
+
+  unsigned char* xw = smem + wave * kWaveBytes;                   // this wave's X' and zeros
+  float* red = reinterpret_cast<float*>(smem + W * kWaveBytes);   // [W][R * MB][64]
+  if (lane < 16) *reinterpret_cast<uint4*>(xw + kXBytes + lane * 16) = make_uint4(0, 0, 0, 0);
+
+  constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
+  const UnpackConsts<BITS> consts;
+  // activation operand: row n of A is batch row n % 4 while tile u = n / 4 of a group of four is
+  // multiplied; the batch rows beyond M repeat row M - 1 (their results are never stored)
+  const int arow = (n & 3) < a.M ? (n & 3) : a.M - 1;
+  const unsigned char* a_live = xw + (MB > 1 ? arow * T * 256 : 0) + q * 16;
+  const unsigned char* a_zero = xw + kXBytes + q * 16;
+
+  float acc[R][MB];
+#pragma unroll
+  for (int rr = 0; rr < R; rr++)
+#pragma unroll
+    for (int v = 0; v < MB; v++) acc[rr][v] = 0.f;
+
+  for (int kt0 = wave * T; kt0 < a.k_tiles; kt0 += W * T) {
+    const int left = a.k_tiles - kt0;
+    const int nt = left < T ? left : T;  // tiles of this round
+
+    // ---- requests, oldest first: activations, scales and zeros, codes.  Every request is
+    // unconditional; what lies past the round is cut off by the size of its descriptor and
+    // reads as zero (zero scale: such a tile adds nothing).
+    u32x4 xv[MB][TH];
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+      const int mrow = m < a.M ? m : a.M - 1;
+      const BufRsrc xr = make_rsrc(a.x + (size_t)mrow * a.K, (uint32_t)(kt0 + nt) * 256u);
+#pragma unroll
+      for (int h = 0; h < TH; h++)
+        xv[m][h] = __builtin_amdgcn_raw_buffer_load_b128(xr, lane * 16, (uint32_t)(kt0 + 4 * h) * 256u, 0);
+    }
+    uint16_t sv[R][TH], zv[R][TH];
+    uint32_t w[R][T][BITS];
+#pragma unroll
+    for (int rr = 0; rr < R; rr++) {
+      const bool rows = rb0 + rr < a.row_blocks;
+      const uint32_t g0 = (uint32_t)(rb0 + rr) * a.k_tiles + kt0;  // first tile = first group
+      const BufRsrc sr = make_rsrc(a.scales, rows ? (g0 + nt) * 32u : 0u);
+      const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, rows ? (g0 + nt) * 32u : 0u);
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        sv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(sr, lane * 2, (g0 + 4 * h) * 32u, 0);
+        if constexpr (ZP) zv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(zr, lane * 2, (g0 + 4 * h) * 32u, 0);
+      }
+    }
+#pragma unroll
+    for (int rr = 0; rr < R; rr++) {
+      const bool rows = rb0 + rr < a.row_blocks;
+      const uint32_t g0 = (uint32_t)(rb0 + rr) * a.k_tiles + kt0;
+      const BufRsrc wr = make_rsrc(a.packed, rows ? (g0 + nt) * tile_bytes : 0u);
+#pragma unroll
+      for (int i = 0; i < T; i++) load_tile_words<BITS>(wr, (g0 + i) * tile_bytes, lane, w[rr][i]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- stage X' = X 2^-p (lane: chunk lane % 16 of tile 4 h + lane / 16) and form the two
+    // sums of every tile; after the rotate-reduce each lane of quarter q holds those of tile 4 h + q
+    float off[MB][TH], xs[MB][TH];
+    const half2v ones = h2_splat(1.0f);
+#pragma unroll
+    for (int m = 0; m < MB; m++) {
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        Frag v;
+        v.v = make_uint4(xv[m][h].x, xv[m][h].y, xv[m][h].z, xv[m][h].w);
+        v.h = storage8_to_half8(v.h);
+        float sx = dot2(v.p[0], ones, 0.f);
+        sx = dot2(v.p[1], ones, sx);
+        sx = dot2(v.p[2], ones, sx);
+        sx = dot2(v.p[3], ones, sx);
+        if constexpr (BITS != 8) {
+          // pair i of octet j is scaled by 2^-p(j, i); only 2-bit codes depend on j (its parity)
+          const bool odd = BITS == 2 && (n & 4) != 0;  // octet = chunk / 4, chunk = lane % 16
+          const float i0 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 0)), i1 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 1));
+          const float i2 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 2)), i3 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 3));
+          const float o0 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 0)), o1 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 1));
+          const float o2 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 2)), o3 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 3));
+          v.p[0] = v.p[0] * h2_splat(odd ? o0 : i0);
+          v.p[1] = v.p[1] * h2_splat(odd ? o1 : i1);
+          v.p[2] = v.p[2] * h2_splat(odd ? o2 : i2);
+          v.p[3] = v.p[3] * h2_splat(odd ? o3 : i3);
+        }
+        float so = dot2(v.p[0], ones, 0.f);
+        so = dot2(v.p[1], ones, so);
+        so = dot2(v.p[2], ones, so);
+        so = dot2(v.p[3], ones, so);
+        if (T >= 4 || 4 * h + q < T)
+          *reinterpret_cast<uint4*>(xw + m * T * 256 + h * 1024 + lane * 16) = v.v;
+        xs[m][h] = row_sum16(sx);
+        off[m][h] = 1024.0f * row_sum16(so);
+      }
+    }
+
+    // ---- the tiles, in request order
+    float4v d[R];
+#pragma unroll
+    for (int rr = 0; rr < R; rr++) d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < T; i++) {
+      const int u = i & 3;
+      const unsigned char* ab = (n >> 2) == u ? a_live + i * 256 : a_zero;
+      Frag av[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) av[j].v = *reinterpret_cast<const uint4*>(ab + j * 64);
+#pragma unroll
+      for (int rr = 0; rr < R; rr++) {
+        Frag bw;
+        raw_octet<BITS, 0>(w[rr][i], consts, bw.u);
+        d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[0].h, bw.h, d[rr], 0, 0, 0);
+        raw_octet<BITS, 1>(w[rr][i], consts, bw.u);
+        d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[1].h, bw.h, d[rr], 0, 0, 0);
+        raw_octet<BITS, 2>(w[rr][i], consts, bw.u);
+        d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[2].h, bw.h, d[rr], 0, 0, 0);
+        raw_octet<BITS, 3>(w[rr][i], consts, bw.u);
+        d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[3].h, bw.h, d[rr], 0, 0, 0);
+      }
+      if (u == 3 || i == T - 1) {
+        const int h = i >> 2;
+#pragma unroll
+        for (int rr = 0; rr < R; rr++) {
+          const float s = storage_to_float(sv[rr][h]);
+          float zs = (float)(1 << (BITS - 1));
+          if constexpr (ZP) zs = storage_to_float(zv[rr][h]) * (1.0f / kMul);
+#pragma unroll
+          for (int v = 0; v < MB; v++) acc[rr][v] += s * (d[rr][v] - off[v][h] - zs * xs[v][h]);
+          d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
+        }
+      }
+    }
+  }
+
+  // ---- the four lane quarters and the W waves meet: red[wave][rr * MB + v][lane]
+#pragma unroll
+  for (int rr = 0; rr < R; rr++)
+#pragma unroll
+    for (int v = 0; v < MB; v++) red[((wave * R + rr) * MB + v) * 64 + lane] = acc[rr][v];
+  __syncthreads();
+  for (int o = wave; o < R * MB; o += W) {
+    float sum = 0.f;
+    for (int w2 = 0; w2 < W; w2++) sum += red[(w2 * R * MB + o) * 64 + lane];
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    const int rr = o / MB, v = o - rr * MB;
+    if (q == 0 && rb0 + rr < a.row_blocks && v < a.M)
+      a.y[(size_t)v * a.N + (size_t)(rb0 + rr) * 16 + n] = float_to_storage(sum * kMul);
+  }
+}
+
+// WPE: waves per SIMD the register allocation is held to
+template <int BITS, bool ZP, int T, int R, int MB, int WPE>
+__global__ void __launch_bounds__(1024, WPE) gemv_kernel(const GemmArgs a, const int W) {
+  gemv_body<BITS, ZP, T, R, MB>(a, W);
+}
+
+template <bool ZP, int T, int R, int MB, int WPE>
+hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stream) {
+  const dim3 grid((a.row_blocks + R - 1) / R), block(64 * W);
+  size_t smem = (size_t)W * gemv_wave_lds(T, MB) + (size_t)W * R * MB * 256;
+  if (smem < lds_pad) smem = lds_pad;
+  if (W < 1 || W > 16 || a.M > MB || smem > 160 * 1024) return hipErrorInvalidValue;
+  if (smem > 64 * 1024) {
+    // more than 64 KiB of dynamic LDS has to be allowed once per kernel
+    static bool allowed = false;
+    if (!allowed) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, T, R, MB, WPE>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return e;
+      allowed = true;
+    }
+  }
+  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, T, R, MB, WPE>), grid, block, smem, stream, a, W);
+  return hipGetLastError();
+}
+
+// shapes built: (T tiles per wave and round, R row blocks per workgroup)
+template <bool ZP, int MB>
+hipError_t launch_shape(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t s) {
+  switch (shape) {
+    case 0: return launch_one<ZP, 8, 1, MB, 4>(a, W, lds_pad, s);
+    case 1: return launch_one<ZP, 4, 1, MB, 4>(a, W, lds_pad, s);
+    case 2: return launch_one<ZP, 4, 2, MB, 4>(a, W, lds_pad, s);
+    case 3: return launch_one<ZP, 2, 2, MB, 4>(a, W, lds_pad, s);
+    case 4: return launch_one<ZP, 2, 4, MB, 4>(a, W, lds_pad, s);
+    default: return launch_one<ZP, 2, 1, MB, 4>(a, W, lds_pad, s);
+  }
+}
+
+}  // namespace
+
+// Entry of this translation unit.  shape: index into the (T, R) table above; W: waves per
+// workgroup (1..16); lds_pad: dynamic LDS to ask for when it exceeds what the kernel needs
+// (limits how many workgroups share a CU).  Group size 128 and M <= 4 only.
+#define MATGPTQ_CAT2(a, b) a##b
+#define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
+#if MATGPTQ_BF16
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(MATGPTQ_CAT(launch_gemv_b, MATGPTQ_BITS), _bf16)
+#else
+#define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_gemv_b, MATGPTQ_BITS)
+#endif
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t stream) {
+  const bool zp = a.zeros != nullptr;
+  if (a.M == 1)
+    return zp ? launch_shape<true, 1>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, 1>(a, shape, W, lds_pad, stream);
+  return zp ? launch_shape<true, 4>(a, shape, W, lds_pad, stream)
+            : launch_shape<false, 4>(a, shape, W, lds_pad, stream);
+}
+
+}  // namespace matgptq

@@ -225,11 +225,12 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 #pragma unroll
     for (int i = 0; i < MB; i++) red[((wave * R + rr) * MB + i) * 64 + lane] = acc[rr][i];
   __syncthreads();
-  if (tid < R * MB * 64) {
-    float4v sum = red[tid];
+  // (R * MB * 64 outputs of four values each: up to twice the threads of the workgroup)
+  for (int ot = tid; ot < R * MB * 64; ot += 64 * kWaves) {
+    float4v sum = red[ot];
 #pragma unroll
-    for (int w = 1; w < kWaves; w++) sum += red[w * R * MB * 64 + tid];
-    const int l = tid & 63, ri = tid >> 6;
+    for (int w = 1; w < kWaves; w++) sum += red[w * R * MB * 64 + ot];
+    const int l = ot & 63, ri = ot >> 6;
     const int rb = rb_first + ri / MB;
     const int m = m0 + (ri % MB) * 16 + (l & 15);
     if (rb < a.row_blocks && m < a.M) {

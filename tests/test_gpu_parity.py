@@ -36,7 +36,7 @@ def test_slice_pack_unpack_bit_exact(b):
     assert np.array_equal(dev.cpu().numpy().view(np.uint32), host)
     assert np.array_equal(G.pack_device(ref, b, from_master=False).cpu().numpy().view(np.uint32), host)
     # the codes the GEMM kernels see (device unpack uses their unpack sequence)
-    back = torch.empty(n, k, dtype=torch.uint8, device=G.DEV)
+    back = torch.full((n, k), 255, dtype=torch.uint8, device=G.DEV)
     _lib.check(L.matgptq_unpack_device(dev.data_ptr(), n, k, b, back.data_ptr(), G.stream()))
     assert np.array_equal(back.cpu().numpy(), ref)
 
@@ -56,7 +56,7 @@ def test_slice_device_odd_length():
 def test_dequantize_bit_exact(b, g, golden):
     L = G.lib()
     lay = G.Layer(48, 512, b, g, seed=10 + b)
-    w = torch.empty(48, 512, dtype=torch.float16, device=G.DEV)
+    w = torch.full((48, 512), float("nan"), dtype=torch.float16, device=G.DEV)
     _lib.check(L.matgptq_dequantize_device(b, g, 48, 512, lay.packed.data_ptr(), lay.scales.data_ptr(),
                                            lay.zeros.data_ptr(), w.data_ptr(), G.stream()))
     assert np.array_equal(w.cpu().numpy().view(np.uint16), lay.w.view(np.uint16))
@@ -64,7 +64,7 @@ def test_dequantize_bit_exact(b, g, golden):
         n, k = golden["q"].shape
         pk = G.pack_device(golden["q"], b, True)
         sd, zd = G.reorder_device(golden["scale"], n, k, g), G.reorder_device(golden["zero"], n, k, g)
-        w = torch.empty(n, k, dtype=torch.float16, device=G.DEV)
+        w = torch.full((n, k), float("nan"), dtype=torch.float16, device=G.DEV)
         _lib.check(L.matgptq_dequantize_device(b, g, n, k, pk.data_ptr(), sd.data_ptr(), zd.data_ptr(),
                                                w.data_ptr(), G.stream()))
         assert np.array_equal(w.cpu().numpy().view(np.uint16), golden[f"w_b{b}"].view(np.uint16))
@@ -313,7 +313,7 @@ def _gemm_bf16(b, g, n, k, x_f32, packed, s_f32, z_f32, flags=3):
         zd = _bf16_dev(z_f32)
         zr = torch.empty_like(zd)
         _lib.check(L.matgptq_reorder_scales_device(zd.data_ptr(), n, k, g, zr.data_ptr(), G.stream()))
-    y = torch.empty(xd.shape[0], n, dtype=torch.bfloat16, device=G.DEV)
+    y = torch.full((xd.shape[0], n), float("nan"), dtype=torch.bfloat16, device=G.DEV)  # poisoned
     _lib.check(L.matgptq_gemm(b, g, n, k, xd.shape[0], packed.data_ptr(), sr.data_ptr(),
                               zr.data_ptr() if zr is not None else None, xd.data_ptr(), y.data_ptr(),
                               G.stream(), flags))
