@@ -11,11 +11,16 @@ Format (what the reference's `pack_quantized_model.py` writes and its vLLM plugi
     (:134-141); generation config and tokenizer files are carried over.
 
 The quantiser's output that goes in is one directory per layer with a `data.pt` holding
-`qweight` and `scale` (:11-22).  Two things are added, both optional and ignored by the
-reference reader: `<layer>.zeros` when `data.pt` has a `zero` (asymmetric quantisation; the
-reference's kernels are symmetric, zero = 128) and `<layer>.perm` when it has a `perm`
-(act-order column permutation), plus a `layer_bitwidths` map in `quantization_config`
-(Mix'n'Match: the per-layer file of inference_demo_transformers.py:58-62 as part of the checkpoint).
+`qweight` and `scale` (:11-22).  Additions, all optional:
+  * `<layer>.zeros` when `data.pt` has a `zero` that is not 128 everywhere (asymmetric
+    quantisation; the reference's packer drops `zero`, :15-18, and its kernels assume 128).
+    `quantization_config.has_zeros` is then true and the plugin of this package registers a
+    `zeros` parameter for every quantised linear; a checkpoint whose zeros are all 128 carries
+    no such tensors and stays readable by the reference's plugin;
+  * `<layer>.perm` when `data.pt` has a `perm` that is not the identity (act-order column
+    permutation, src/mat_gptq.py:155-159); `quantization_config.has_perm` is then true;
+  * a `layer_bitwidths` map in `quantization_config` (Mix'n'Match: the per-layer file of
+    inference_demo_transformers.py:58-62 as part of the checkpoint).
 
 Unlike the reference script this one needs neither `transformers` nor the model class:
 `config.json` is edited as JSON and the tokenizer files are copied.  `data.pt` files are
@@ -47,12 +52,13 @@ CARRIED_FILES = ("generation_config.json", "tokenizer.json", "tokenizer_config.j
                  "chat_template.jinja")
 
 
-def load_quantised_layer(layer_dir: str) -> Dict[str, torch.Tensor]:
-    """`qweight`, `scale` (and `zero`, `perm` when stored) of one layer (pack_quantized_model.py:11-22)."""
+def load_quantised_layer(layer_dir: str, mmap: bool = False) -> Dict[str, torch.Tensor]:
+    """`qweight`, `scale` (and `zero`, `perm` when stored) of one layer (pack_quantized_model.py:11-22).
+    With `mmap` the tensors are mapped from the file and read only where they are touched."""
     data_pt = os.path.join(layer_dir, "data.pt")
     if not os.path.exists(data_pt):
         raise FileNotFoundError(f"No data.pt found in {layer_dir}")
-    data = torch.load(data_pt, map_location="cpu", weights_only=True)
+    data = torch.load(data_pt, map_location="cpu", weights_only=True, mmap=mmap)
     out = {"qweight": data["qweight"], "scale": data["scale"]}
     for key in ("zero", "perm"):
         if data.get(key) is not None:
@@ -101,8 +107,17 @@ def _packed_tensors(name: str, q: Dict[str, torch.Tensor], group_size: int,
     if "zero" in q:
         out[f"{name}.zeros"] = q["zero"].cpu().reshape(n, -1).to(out[f"{name}.scales"].dtype).contiguous()
     if "perm" in q:
-        out[f"{name}.perm"] = q["perm"].cpu().to(torch.int32).contiguous()
+        out[f"{name}.perm"] = q["perm"].cpu().to(torch.int32).reshape(-1).contiguous()
     return out
+
+
+def _all_symmetric(zero: torch.Tensor) -> bool:
+    return bool((zero.float() == 128.0).all())
+
+
+def _is_identity(perm: torch.Tensor) -> bool:
+    perm = perm.reshape(-1).to(torch.int64)
+    return bool((perm == torch.arange(perm.numel())).all())
 
 
 def pack_model(model_name_or_path: str, quantised_dir: str, output_dir: str, group_size: int,
@@ -120,6 +135,16 @@ def pack_model(model_name_or_path: str, quantised_dir: str, output_dir: str, gro
     quantised_layers = {name for name in os.listdir(quantised_dir)
                         if os.path.isdir(os.path.join(quantised_dir, name))}
     new_weight_map: Dict[str, str] = {}
+    if not os.path.exists(index_path) and not os.path.exists(single_path):
+        raise FileNotFoundError(f"Neither {INDEX_NAME} nor {SINGLE_NAME} found.")
+    # One rule for the whole checkpoint, because the plugin registers the same parameters for
+    # every quantised linear: zeros are written for all layers or for none, and so is perm.
+    packable = sorted(name for name in quantised_layers if not should_skip_quantisation(name))
+    has_zeros = has_perm = False
+    for layer in packable:
+        q = load_quantised_layer(os.path.join(quantised_dir, layer), mmap=True)  # the codes stay on disk
+        has_zeros = has_zeros or ("zero" in q and not _all_symmetric(q["zero"]))
+        has_perm = has_perm or ("perm" in q and not _is_identity(q["perm"]))
 
     def convert(shard_name: str, names, tensors) -> None:
         new_tensors: Dict[str, torch.Tensor] = {}
@@ -131,6 +156,14 @@ def pack_model(model_name_or_path: str, quantised_dir: str, output_dir: str, gro
                 layer = t_name.rsplit(".", 1)[0]
                 if layer in quantised_layers and not should_skip_quantisation(layer):
                     q = load_quantised_layer(os.path.join(quantised_dir, layer))
+                    if has_zeros:
+                        q.setdefault("zero", torch.full_like(q["scale"], 128.0))
+                    else:
+                        q.pop("zero", None)
+                    if has_perm:
+                        q.setdefault("perm", torch.arange(q["qweight"].shape[1]))
+                    else:
+                        q.pop("perm", None)
                     for key, value in _packed_tensors(layer, q, group_size, dtype).items():
                         new_tensors[key] = value
                         new_weight_map[key] = shard_name
@@ -147,11 +180,9 @@ def pack_model(model_name_or_path: str, quantised_dir: str, output_dir: str, gro
             convert(shard_name, [t for t, s in original_map.items() if s == shard_name], tensors)
         with open(os.path.join(output_dir, INDEX_NAME), "w") as f:
             json.dump({"metadata": {}, "weight_map": new_weight_map}, f)
-    elif os.path.exists(single_path):
+    else:
         tensors = load_file(single_path)
         convert(SINGLE_NAME, list(tensors.keys()), tensors)
-    else:
-        raise FileNotFoundError(f"Neither {INDEX_NAME} nor {SINGLE_NAME} found.")
 
     config_path = os.path.join(model_name_or_path, "config.json")
     config = {}
@@ -166,6 +197,10 @@ def pack_model(model_name_or_path: str, quantised_dir: str, output_dir: str, gro
         "quant_method": QUANT_METHOD,
         "quant_dtype": quant_dtype,
     }
+    if has_zeros:
+        quantization_config["has_zeros"] = True
+    if has_perm:
+        quantization_config["has_perm"] = True
     if layer_bitwidths:
         quantization_config["layer_bitwidths"] = dict(layer_bitwidths)
     config["quantization_config"] = quantization_config
@@ -233,8 +268,8 @@ def bitwidth_of(layer: str, quantization_config: dict) -> int:
 def build_linear(tensors: Dict[str, torch.Tensor], bitwidth: int, quantization_config: dict,
                  device: str = "cuda"):
     """A `MatGPTQLinear` for one layer of a packed checkpoint: slice to `bitwidth`, pack,
-    reorder (inference_demo_transformers.py:30-40).  A stored column permutation is applied
-    to the input features by the returned module's caller: `x[..., perm]`."""
+    reorder (inference_demo_transformers.py:30-40).  A stored column permutation becomes part
+    of the module, which gathers its input features with it (`x[..., perm]`)."""
     from matgptq_cuda.matgptq_linear import MatGPTQLinear
 
     from .ops import matryoshka_slice
@@ -242,9 +277,11 @@ def build_linear(tensors: Dict[str, torch.Tensor], bitwidth: int, quantization_c
     master = quantization_config["master_bitwidth"]
     q = tensors["qweight"].to(device)
     zeros = tensors.get("zeros")
+    perm = tensors.get("perm")
     return MatGPTQLinear(matryoshka_slice(q, master, bitwidth), tensors["scales"].to(device), bitwidth,
                          quantization_config["group_size"],
-                         zeros=zeros.to(device) if zeros is not None else None)
+                         zeros=zeros.to(device) if zeros is not None else None,
+                         perm=perm.to(device) if perm is not None else None)
 
 
 def main() -> None:

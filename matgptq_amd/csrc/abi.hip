@@ -252,10 +252,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     p->smem = 0;
     return MATGPTQ_OK;
   }
-  // burst keeps at most eight waves per workgroup; long tile runs prefer stream
-  const int tiles_per_wave = (k_tiles + W - 1) / W * R;
-  bool stream = flavour == 2 || (flavour == 0 && S * W > 8);
-  (void)tiles_per_wave;
+  // burst keeps at most eight waves per workgroup
+  const bool stream = flavour == 2 || (flavour == 0 && S * W > 8);
   if (!stream && S * W > 8) return MATGPTQ_EVARIANT;
   // largest kc whose activations fit next to the partial sums and scales
   const int64_t fixed = (int64_t)decode_lds_bytes(R, S, W, 0, 0);

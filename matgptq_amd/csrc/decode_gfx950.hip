@@ -273,12 +273,6 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
     using J1 = std::integral_constant<int, 1>;
     using J2 = std::integral_constant<int, 2>;
     using J3 = std::integral_constant<int, 3>;
-#ifdef MATGPTQ_DEBUG_NOCOMPUTE
-    for (int rr = 0; rr < R; rr++)
-      for (int j = 0; j < BITS; j++) acc[rr][0] += __uint_as_float(st.w[u][rr][j] & 0x3f000000u);
-    if (tl < 0) acc[0][1] += (float)xb[tl];
-    return;
-#endif
     Frag b[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) b[j].v = *reinterpret_cast<const uint4*>(xb + tl * 128 + j * 32);
@@ -432,10 +426,6 @@ __device__ __forceinline__ void decode_body(const GemmArgs& a, const DecodeShape
     }
   }
 
-#ifdef MATGPTQ_DEBUG_NOREDUCE
-  if (acc[0][0] == 1.2345f) a.y[tid] = 1;
-  return;
-#endif
   // combine the W partial sums of each slot: red[wave][rr][lane*4 + i]
 #pragma unroll
   for (int rr = 0; rr < R; rr++)

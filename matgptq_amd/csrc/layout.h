@@ -35,7 +35,7 @@
 #pragma once
 #include <stdint.h>
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define MATGPTQ_HD __host__ __device__ __forceinline__
 #else
 #define MATGPTQ_HD inline

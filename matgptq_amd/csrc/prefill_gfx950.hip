@@ -112,11 +112,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
       const int rb = rb_first + rr;
-#ifdef MATGPTQ_DEBUG_NOWLOAD
-      const bool valid = rb < a.row_blocks && kb == 0;
-#else
       const bool valid = rb < a.row_blocks && kb < a.k_tiles;
-#endif
       const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
       const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
       const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
@@ -146,11 +142,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     x_lds[c] = (uint32_t)(row * kXsPitch + col8 * 8);
   }
   auto load_x = [&](u32x4 (&xr)[XCHUNKS], int h) {  // columns [h*64, +64)
-#ifdef MATGPTQ_DEBUG_NOXLOAD
-    const bool valid = h < 0;
-#else
     const bool valid = h < 2 * a.k_tiles;
-#endif
     const BufRsrc xres = make_rsrc(a.x, valid ? x_bytes : 0u);
 #pragma unroll
     for (int c = 0; c < XCHUNKS; c++)
@@ -182,12 +174,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       }
       const half2v sc = {s1, s1};
       const half2v zr = {z1, z1};
-#ifdef MATGPTQ_DEBUG_NODEQUANT
-      aw[rr].u[0] = w[rr][0]; aw[rr].u[1] = w[rr][1 % BITS]; aw[rr].u[2] = w[rr][0] ^ J; aw[rr].u[3] = w[rr][1 % BITS];
-      (void)sc; (void)zr;
-#else
       dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
-#endif
     }
   };
   auto read_frag = [&](Frag& b, int i, int buf, int jj) {

@@ -151,7 +151,9 @@ Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& sca
   TORCH_CHECK(scales.dtype() == want, "matmul_matgptq: matgptq_scales must be ", want_name);
   TORCH_CHECK(input.dim() >= 2 && input.size(-1) == n_in_features,
               "matmul_matgptq: input must be (..., batch, n_in_features)");
-  TORCH_CHECK(input.is_contiguous(), "matmul_matgptq: input must be contiguous");
+  // the reference reads the input as if it were contiguous (bindings.cpp:171-186): a strided
+  // view (a slice of a fused projection, a transposed batch) is compacted first
+  const Tensor input_c = input.contiguous();
   const int64_t groups = group_size == -1 ? 1 : n_in_features / group_size;
   TORCH_CHECK(scales.is_contiguous() && scales.numel() == n_out_features * groups,
               "matgptq_scales has the wrong size");
@@ -174,7 +176,7 @@ Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& sca
   if (m == 0) return out;
   const uint32_t flags = (uint32_t)feature_flag | MATGPTQ_FLAG_ASYNC;
   const int code = matgptq_gemm((int)bitwidth, (int)group_size, n_out_features, n_in_features, m,
-                                weights.data_ptr(), scales.data_ptr(), zeros_ptr, input.data_ptr(),
+                                weights.data_ptr(), scales.data_ptr(), zeros_ptr, input_c.data_ptr(),
                                 out.data_ptr(), stream_of(dev), flags);
   check_abi(code, "matmul_matgptq");
   if (!(feature_flag & MATGPTQ_FLAG_ASYNC)) {

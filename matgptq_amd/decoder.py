@@ -44,16 +44,19 @@ def replace_with_matgptq_linear(model: torch.nn.Module, quantized_weights_path: 
     With `quantized_config_path` (lines `layer_name: bitwidth`, as written by the reference's
     search, evo_quant_search.py:660-672) exactly the listed layers are replaced, each at its own
     bitwidth; without it every layer directory is replaced at `slice_bitwidth`.  A stored
-    `zero` tensor is used when present (the reference drops it and assumes 128).
+    `zero` tensor is used when present (the reference drops it and assumes 128), and a stored
+    act-order `perm` is applied to the module's input features (the reference's kernel path
+    ignores it; its fake-quantised path applies it, src/model_utils.py:185-195).
     """
     from matgptq_cuda.matgptq_linear import MatGPTQLinear
 
     def _replace(layer_name: str, bitwidth: int) -> None:
         data = load_quantised_layer(os.path.join(quantized_weights_path, layer_name))
         codes = matryoshka_slice(data["qweight"].cuda(), master_bitwidth, bitwidth)
-        zero = data.get("zero")
+        zero, perm = data.get("zero"), data.get("perm")
         layer = MatGPTQLinear(codes, data["scale"].cuda(), bitwidth, group_size,
-                              zeros=zero.cuda() if zero is not None else None)
+                              zeros=zero.cuda() if zero is not None else None,
+                              perm=perm.cuda() if perm is not None else None)
         *parent_path, attr = layer_name.split(".")
         parent = model.get_submodule(".".join(parent_path)) if parent_path else model
         setattr(parent, attr, layer)

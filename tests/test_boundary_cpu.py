@@ -111,5 +111,5 @@ def test_plugin_create_weights_shapes_and_alignment_error():
     assert (layer.qweight.input_dim, layer.qweight.output_dim) == (1, 0)
     assert layer.scales.shape == (48, 2) and layer.scales.dtype == torch.float16
     assert (layer.scales.input_dim, layer.scales.output_dim, layer.scales.packed_dim) == (1, 0, 1)
-    with pytest.raises(ValueError, match="not aligned"):
+    with pytest.raises(ValueError, match="not a multiple of the quantisation group size"):
         m.create_weights(torch.nn.Module(), 200, [32], 200, 32, torch.float16)

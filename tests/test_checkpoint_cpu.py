@@ -116,6 +116,9 @@ def test_pack_model_writes_the_reference_format(tmp_path, sharded, with_extras):
     c = vllm_matgptq.MatGPTQConfig.from_config(qc)
     assert c.inference_bitwidth == 4 and c.group_size == 128
     assert c.bitwidth_for(LAYERS[0]) == (3 if with_extras else 4)
+    # zeros / perm are announced in the config exactly when the shards carry them
+    assert qc.get("has_zeros", False) == with_extras and qc.get("has_perm", False) == with_extras
+    assert c.has_zeros == with_extras and c.has_perm == with_extras
 
     # reader
     assert ck.read_quantization_config(out) == qc
@@ -151,3 +154,79 @@ def test_layer_bitwidth_file(tmp_path):
     assert ck.read_layer_bitwidths(str(p)) == {LAYERS[0]: 3, LAYERS[1]: 6}
     assert np.all([not ck.should_skip_quantisation(x) for x in LAYERS])
     assert ck.should_skip_quantisation("lm_head") and ck.should_skip_quantisation("model.norm")
+
+
+def test_symmetric_zeros_and_identity_perm_are_not_written(tmp_path):
+    # the reference quantiser always stores a `zero` (128 everywhere for symmetric recipes) and its
+    # plugin registers only qweight and scales: such a checkpoint must not carry tensors a loader
+    # has no parameter for
+    model, quant, out = str(tmp_path / "m"), str(tmp_path / "q"), str(tmp_path / "out")
+    _make_model(model, False)
+    os.makedirs(quant)
+    for i, (name, (n, k)) in enumerate({LAYERS[0]: (32, 128), LAYERS[1]: (16, 256)}.items()):
+        q, s, _ = o.make_layer(n, k, 128, seed=i)
+        os.makedirs(os.path.join(quant, name))
+        torch.save({"qweight": torch.from_numpy(q), "scale": torch.from_numpy(s),
+                    "zero": torch.full((n, k // 128), 128.0).half(), "perm": torch.arange(k)},
+                   os.path.join(quant, name, "data.pt"))
+    wm = ck.pack_model(model, quant, out, 128, 8, 4, "float16")
+    assert not any(name.endswith((".zeros", ".perm")) for name in wm)
+    qc = ck.read_quantization_config(out)
+    assert "has_zeros" not in qc and "has_perm" not in qc
+
+
+def test_mixed_layers_get_zeros_everywhere(tmp_path):
+    # one asymmetric layer makes the checkpoint asymmetric: every quantised linear then carries
+    # zeros (128 where the quantiser stored none), because the plugin registers them per config
+    model, quant, out = str(tmp_path / "m"), str(tmp_path / "q"), str(tmp_path / "out")
+    _make_model(model, False)
+    os.makedirs(quant)
+    q0, s0, z0 = o.make_layer(32, 128, 128, seed=0)
+    q1, s1, _ = o.make_layer(16, 256, 128, seed=1)
+    for name, data in ((LAYERS[0], {"qweight": q0, "scale": s0, "zero": z0}), (LAYERS[1], {"qweight": q1, "scale": s1})):
+        os.makedirs(os.path.join(quant, name))
+        torch.save({k: torch.from_numpy(v) for k, v in data.items()}, os.path.join(quant, name, "data.pt"))
+    wm = ck.pack_model(model, quant, out, 128, 8, 4, "float16")
+    got = load_file(os.path.join(out, ck.SINGLE_NAME))
+    assert torch.equal(got[f"{LAYERS[0]}.zeros"], torch.from_numpy(z0))
+    assert torch.equal(got[f"{LAYERS[1]}.zeros"], torch.full((16, 2), 128.0).half())
+    assert ck.read_quantization_config(out)["has_zeros"] is True and f"{LAYERS[1]}.perm" not in wm
+
+
+def _strict_load(layer: torch.nn.Module, tensors: dict) -> None:
+    """What a model loader does with a layer's tensors: every name must have a registered
+    parameter of the same shape and dtype; unknown names are an error."""
+    params = dict(layer.named_parameters())
+    for name, t in tensors.items():
+        if name not in params:
+            raise KeyError(f"unexpected tensor {name}")
+        assert params[name].shape == t.shape and params[name].dtype == t.dtype, name
+        params[name].data.copy_(t)
+
+
+@pytest.mark.parametrize("with_extras", (False, True))
+def test_plugin_registers_what_the_checkpoint_carries(tmp_path, with_extras):
+    model, quant, out = str(tmp_path / "m"), str(tmp_path / "q"), str(tmp_path / "out")
+    _make_model(model, False)
+    _make_quantised(quant, with_extras)
+    ck.pack_model(model, quant, out, 128, 8, 4, "float16")
+    qc = ck.read_quantization_config(out)
+    config = vllm_matgptq.MatGPTQConfig.from_config(qc)
+    for name, tensors in ck.iter_quantised_layers(out):
+        n, k = tensors["qweight"].shape
+        layer = torch.nn.Module()
+        method = vllm_matgptq.MatGPTQLinearMethod(config, config.bitwidth_for(name))
+        method.create_weights(layer, k, [n], k, n, torch.float16)
+        assert set(dict(layer.named_parameters())) == set(tensors)
+        _strict_load(layer, tensors)
+    # a config without the flags registers neither, and the same tensors are then refused
+    plain = vllm_matgptq.MatGPTQConfig.from_config({k: v for k, v in qc.items() if k not in ("has_zeros", "has_perm")})
+    layer = torch.nn.Module()
+    vllm_matgptq.MatGPTQLinearMethod(plain).create_weights(layer, 128, [32], 128, 32, torch.float16)
+    assert set(dict(layer.named_parameters())) == {"qweight", "scales"}
+    if with_extras:
+        with pytest.raises(KeyError, match="unexpected tensor"):
+            _strict_load(layer, dict(ck.iter_quantised_layers(out))[LAYERS[0]])
+        # act-order and a split of in_features do not go together
+        with pytest.raises(ValueError, match="act-order"):
+            vllm_matgptq.MatGPTQLinearMethod(config).create_weights(torch.nn.Module(), 128, [32], 256, 32, torch.float16)

@@ -231,3 +231,153 @@ def test_mixnmatch_stack_through_plugin():
         G.assert_close_to_oracle(y.cpu().numpy(), x, w, f"{name} b={bits[name]}")
     assert isinstance(cfg.get_quant_method(vllm_matgptq.LinearBase(), "lm_head"),
                       vllm_matgptq.UnquantizedLinearMethod)
+
+
+def test_act_order_permutation_is_applied():
+    # FakeMatryoshkaLinear.forward gathers the input features with `perm` before the product
+    # (src/quant_utils_matgpqt.py:218-220): the codes are stored in permuted column order
+    n, k, g, b = 64, 1024, 128, 4
+    q, s, z = o.make_layer(n, k, g, seed=31)
+    perm = np.random.default_rng(3).permutation(k)
+    w = o.dequantize(q, s, z, b, g)
+    lin = MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)), torch.from_numpy(s), b, g,
+                        zeros=torch.from_numpy(z), perm=torch.from_numpy(perm))
+    plain = MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)), torch.from_numpy(s), b, g, zeros=torch.from_numpy(z))
+    for m in (1, 3, 40):
+        x = o.make_activations(m, k, seed=m)
+        y = lin(torch.from_numpy(x).cuda()).cpu().numpy()
+        G.assert_close_to_oracle(y, x[:, perm], w, f"perm M={m}")
+        # equivalently: the dense weight with its columns put back (src/model_utils.py:185-195)
+        G.assert_close_to_oracle(y, x, w[:, np.argsort(perm)], f"perm, dense form M={m}")
+        assert not np.allclose(y, plain(torch.from_numpy(x).cuda()).cpu().numpy(), rtol=1e-2, atol=1e-2)
+    with pytest.raises(ValueError, match="n_in_features"):
+        MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)), torch.from_numpy(s), b, g, perm=torch.arange(k - 1))
+
+
+def test_plugin_loads_an_act_order_asymmetric_checkpoint(tmp_path):
+    # packed checkpoint with zeros and perm -> create_weights -> a loader that refuses unknown
+    # names -> process_weights_after_loading -> apply, against the oracle; build_linear agrees
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    from matgptq_amd import checkpoint as ck
+
+    model, quant, out = str(tmp_path / "m"), str(tmp_path / "q"), str(tmp_path / "out")
+    os.makedirs(model)
+    shapes = {"model.layers.0.mlp.up_proj": (64, 512), "model.layers.0.mlp.down_proj": (48, 1024)}
+    save_file({f"{k}.weight": torch.zeros(n, kk).half() for k, (n, kk) in shapes.items()},
+              os.path.join(model, ck.SINGLE_NAME))
+    with open(os.path.join(model, "config.json"), "w") as f:
+        json.dump({}, f)
+    layers = {}
+    rng = np.random.default_rng(1)
+    for i, (name, (n, k)) in enumerate(shapes.items()):
+        q, s, z = o.make_layer(n, k, 128, seed=50 + i)
+        perm = rng.permutation(k)
+        os.makedirs(os.path.join(quant, name))
+        torch.save({"qweight": torch.from_numpy(q), "scale": torch.from_numpy(s), "zero": torch.from_numpy(z),
+                    "perm": torch.from_numpy(perm)}, os.path.join(quant, name, "data.pt"))
+        layers[name] = (q, s, z, perm)
+    ck.pack_model(model, quant, out, 128, 8, 4, "float16", layer_bitwidths={"down_proj": 3})
+    qc = ck.read_quantization_config(out)
+    assert qc["has_zeros"] and qc["has_perm"]
+    config = vllm_matgptq.MatGPTQConfig.from_config(qc)
+    for name, tensors in ck.iter_quantised_layers(out):
+        q, s, z, perm = layers[name]
+        n, k = q.shape
+        bits = config.bitwidth_for(name)
+        layer = torch.nn.Module()
+        method = vllm_matgptq.MatGPTQLinearMethod(config, bits)
+        method.create_weights(layer, k, [n], k, n, torch.float16)
+        layer.cuda()
+        params = dict(layer.named_parameters())
+        for key, t in tensors.items():
+            assert key in params, f"the loader has no destination for {key}"
+            params[key].data.copy_(t)
+        method.process_weights_after_loading(layer)
+        assert not hasattr(layer, "qweight") and not hasattr(layer, "perm") and not hasattr(layer, "zeros")
+        w = o.dequantize(q, s, z, bits, 128)
+        x = o.make_activations(5, k, seed=bits)
+        y = method.apply(layer, torch.from_numpy(x).cuda())
+        G.assert_close_to_oracle(y.cpu().numpy(), x[:, perm], w, name)
+        y2 = ck.build_linear(tensors, bits, qc)(torch.from_numpy(x).cuda())
+        assert torch.equal(y, y2)
+
+
+def test_resident_master_codes_switch_bitwidth_at_run_time():
+    # the reference deletes the master codes after loading (inference_lib/vllm_matgptq.py:177-178);
+    # kept resident, a layer moves between bitwidths without the checkpoint
+    n, k = 96, 1024
+    q, s, z = o.make_layer(n, k, 128, seed=77)
+    config = vllm_matgptq.MatGPTQConfig(128, 8, 4, "float16", None, keep_master_codes=True)
+    layer = torch.nn.Module()
+    method = vllm_matgptq.MatGPTQLinearMethod(config)
+    method.create_weights(layer, k, [n], k, n, torch.float16)
+    layer.cuda()
+    layer.qweight.data.copy_(torch.from_numpy(q))
+    layer.scales.data.copy_(torch.from_numpy(s))
+    layer.zeros = torch.nn.Parameter(torch.from_numpy(z).cuda(), requires_grad=False)
+    method.process_weights_after_loading(layer)
+    assert torch.equal(layer.matgptq_master.cpu(), torch.from_numpy(q))
+    x = o.make_activations(3, k, seed=5)
+    xd = torch.from_numpy(x).cuda()
+    for bits in (4, 2, 8, 3, 6, 4):
+        method.set_bitwidth(layer, bits)
+        assert layer.matgptq_weights.numel() == bits * n * k // 32
+        G.assert_close_to_oracle(method.apply(layer, xd).cpu().numpy(), x, o.dequantize(q, s, z, bits, 128), f"b={bits}")
+        codes = torch.ops.matgptq_cuda.unpack_matgptq_qweights(layer.matgptq_weights, n, k, bits)
+        assert np.array_equal(codes.cpu().numpy(), o.slice_codes(q, bits))
+    with pytest.raises(ValueError):
+        method.set_bitwidth(layer, 5)
+    plain = vllm_matgptq.MatGPTQLinearMethod(vllm_matgptq.MatGPTQConfig(128, 8, 4, "float16", None))
+    with pytest.raises(RuntimeError, match="keep_master_codes"):
+        plain.set_bitwidth(torch.nn.Module(), 4)
+
+
+def test_strided_input_is_accepted():
+    # the reference never checks the layout of its input (bindings.cpp:146-191)
+    n, k, b = 64, 512, 4
+    q, s, z = o.make_layer(n, k, 128, seed=8)
+    lin = MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)), torch.from_numpy(s), b, 128, zeros=torch.from_numpy(z))
+    x = o.make_activations(6, 2 * k, seed=1)
+    xd = torch.from_numpy(x).cuda()
+    y = lin(xd[:, :k])  # a slice of a wider tensor: row stride 2k
+    G.assert_close_to_oracle(y.cpu().numpy(), x[:, :k], o.dequantize(q, s, z, b, 128), "strided input")
+
+
+@pytest.mark.parametrize("mode", ("default", "reduce-overhead"))
+def test_torch_compile_fullgraph(mode):
+    # how the reference's callers run decode (inference_lib/inference_demo_transformers.py:161-162,
+    # bench_matgptq_matmul.py:48): torch.compile(fullgraph=True) over modules that contain the
+    # operator, which needs nothing but its fake implementation
+    n, k, b = 256, 1024, 4
+    q, s, z = o.make_layer(n, k, 128, seed=4)
+
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = MatGPTQLinear(torch.from_numpy(o.slice_codes(q, b)), torch.from_numpy(s), b, 128,
+                                    zeros=torch.from_numpy(z))
+            self.sym = MatGPTQLinear(torch.from_numpy(o.slice_codes(q[:, :256].copy(), 3)), torch.from_numpy(s[:, :2].copy()), 3, 128)
+
+        def forward(self, x):
+            h = torch.nn.functional.silu(self.up(x))
+            return h + self.sym(h)
+
+    mod = Mlp().cuda()
+    x = torch.from_numpy(o.make_activations(1, k, seed=2)).cuda()
+    eager = mod(x)
+    try:
+        compiled = torch.compile(mod, fullgraph=True, mode=mode)
+        got = [compiled(x).clone() for _ in range(4)]  # warm-up, capture and replays
+    except Exception as e:  # the inductor toolchain (a C++ compiler for its wrapper) may be absent
+        if "fullgraph" in str(e).lower() or "graph break" in str(e).lower():
+            raise
+        compiled = torch.compile(mod, fullgraph=True, backend="aot_eager")
+        got = [compiled(x).clone() for _ in range(2)]
+    torch.cuda.synchronize()
+    for g in got:
+        assert torch.allclose(g, eager, rtol=1e-3, atol=1e-3)
+    G.assert_close_to_oracle(mod.up(x).cpu().numpy(), x.cpu().numpy(), o.dequantize(q, s, z, b, 128), "compiled module's linear")

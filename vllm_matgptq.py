@@ -14,7 +14,14 @@ Differences, all additive:
     already there (the reference copies them to the host and back);
   * optional key `layer_bitwidths` {prefix-suffix: bits} selects a bitwidth per layer
     (Mix'n'Match); layers not listed use `inference_bitwidth`;
-  * optional layer parameter `zeros` [N, K/group_size]: asymmetric checkpoints.
+  * optional keys `has_zeros` / `has_perm`: the checkpoint carries `<layer>.zeros`
+    [N, K/group_size] (asymmetric quantisation) / `<layer>.perm` [K] (act-order) for every
+    quantised linear, and `create_weights` registers parameters of those names so that the
+    loader finds a destination for them.  Without the keys neither is registered, as in the
+    reference.  vLLM is not importable in this build's environment: what its loader does with
+    these parameters is exercised only through a stand-in loader in the tests;
+  * `keep_master_codes` (constructor argument / config key, default false): the 8-bit master
+    codes stay resident after loading and `set_bitwidth` re-slices a layer in place.
 
 vLLM itself is imported lazily: without it the module still imports (the classes then
 derive from small local bases), which is what the CPU test-suite exercises.
@@ -93,6 +100,9 @@ class MatGPTQConfig(QuantizationConfig):
         quant_dtype: str = "float16",
         modules_to_not_convert: Optional[List[str]] = None,
         layer_bitwidths: Optional[Dict[str, int]] = None,
+        has_zeros: bool = False,
+        has_perm: bool = False,
+        keep_master_codes: bool = False,
     ) -> None:
         super().__init__()
         assert group_size in [-1, 32, 128]
@@ -105,6 +115,9 @@ class MatGPTQConfig(QuantizationConfig):
         self.quant_dtype = dtype_map.get(quant_dtype, torch.float16)
         self.modules_to_not_convert = modules_to_not_convert
         self.layer_bitwidths = dict(layer_bitwidths or {})
+        self.has_zeros = bool(has_zeros)
+        self.has_perm = bool(has_perm)
+        self.keep_master_codes = bool(keep_master_codes)
         for bits in [inference_bitwidth, *self.layer_bitwidths.values()]:
             if bits not in (2, 3, 4, 6, 8):
                 raise ValueError("bitwidth must be one of {2, 3, 4, 6, 8}")
@@ -136,7 +149,8 @@ class MatGPTQConfig(QuantizationConfig):
         quant_dtype = cls.get_from_keys(config, ["quant_dtype"])
         layer_bitwidths = config.get("layer_bitwidths")
         return cls(group_size, master_bitwidth, inference_bitwidth, quant_dtype,
-                   modules_to_not_convert, layer_bitwidths)
+                   modules_to_not_convert, layer_bitwidths, config.get("has_zeros", False),
+                   config.get("has_perm", False), config.get("keep_master_codes", False))
 
     def bitwidth_for(self, prefix: str) -> int:
         """Bitwidth of the layer called `prefix`: the longest matching suffix key of
@@ -170,9 +184,9 @@ class MatGPTQLinearMethod(LinearMethodBase):
         group = self.config.group_size if self.config.group_size != -1 else input_size_per_partition
         if input_size_per_partition % group != 0:
             raise ValueError(
-                "The input size is not aligned with the quantized "
-                "weight shape. This can be caused by too large "
-                "tensor parallel size. Or other skill issues.")
+                f"in_features per partition ({input_size_per_partition}) is not a multiple of the "
+                f"quantisation group size ({group}); a tensor-parallel degree that splits K inside "
+                "a group cannot be served")
 
         self.n_out_features = sum(output_partition_sizes)
         self.n_in_features = input_size_per_partition
@@ -194,20 +208,37 @@ class MatGPTQLinearMethod(LinearMethodBase):
                          | extra_weight_attrs)
         layer.register_parameter("scales", scales)
 
+        if self.config.has_zeros:
+            # same shape, sharding and loader as the scales; 128 wherever the loader writes nothing
+            zeros = Parameter(torch.full_like(scales.data, 128.0), requires_grad=False)
+            set_weight_attrs(zeros, {"input_dim": 1, "output_dim": 0, "packed_dim": 1, "pack_factor": 1}
+                             | extra_weight_attrs)
+            layer.register_parameter("zeros", zeros)
+        if self.config.has_perm:
+            if input_size_per_partition != input_size:
+                raise ValueError(
+                    "an act-order checkpoint (has_perm) permutes all input features of a layer; a "
+                    "tensor-parallel degree that splits in_features cannot be served")
+            perm = Parameter(torch.arange(input_size, dtype=torch.int32), requires_grad=False)
+            set_weight_attrs(perm, {"input_dim": 0} | extra_weight_attrs)
+            layer.register_parameter("perm", perm)
+
+    def _pack_at(self, layer: torch.nn.Module, qweight: torch.Tensor, bitwidth: int) -> torch.Tensor:
+        if qweight.is_cuda and self.config.master_bitwidth == 8:
+            # slice and pack in one pass over the master codes, on the GPU
+            return torch.ops.matgptq_cuda.pack_matgptq_master(
+                qweight.contiguous(), self.n_out_features, self.n_in_features, bitwidth,
+                self.config.group_size, self.config.flag)
+        return torch.ops.matgptq_cuda.pack_matgptq_qweights(
+            matryoshka_slice(qweight, self.config.master_bitwidth, bitwidth).contiguous(),
+            self.n_out_features, self.n_in_features, bitwidth,
+            self.config.group_size, self.config.flag)
+
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         with torch.no_grad():
             qweight = layer.qweight.data
-            if qweight.is_cuda and self.config.master_bitwidth == 8:
-                # slice and pack in one pass over the master codes, on the GPU
-                packed = torch.ops.matgptq_cuda.pack_matgptq_master(
-                    qweight.contiguous(), self.n_out_features, self.n_in_features, self.bitwidth,
-                    self.config.group_size, self.config.flag)
-            else:
-                packed = torch.ops.matgptq_cuda.pack_matgptq_qweights(
-                    matryoshka_slice(qweight, self.config.master_bitwidth, self.bitwidth).contiguous(),
-                    self.n_out_features, self.n_in_features, self.bitwidth,
-                    self.config.group_size, self.config.flag)
-            layer.matgptq_weights = Parameter(packed, requires_grad=False)
+            layer.matgptq_weights = Parameter(self._pack_at(layer, qweight, self.bitwidth), requires_grad=False)
+            layer.matgptq_bitwidth = self.bitwidth
             layer.matgptq_scales = Parameter(
                 torch.ops.matgptq_cuda.reorder_matgptq_scales(
                     layer.scales.data.contiguous(), self.n_out_features, self.n_in_features,
@@ -223,21 +254,50 @@ class MatGPTQLinearMethod(LinearMethodBase):
                 del layer.zeros
             else:
                 layer.matgptq_zeros = None
+            perm = getattr(layer, "perm", None)
+            if perm is not None:
+                # act-order: the codes are stored in permuted column order and the input features
+                # are gathered with the permutation (src/quant_utils_matgpqt.py:218-220)
+                layer.matgptq_perm = Parameter(perm.data.to(device=layer.matgptq_weights.device,
+                                                            dtype=torch.int64).reshape(-1), requires_grad=False)
+                del layer.perm
+            else:
+                layer.matgptq_perm = None
 
+            if self.config.keep_master_codes:
+                # The reference deletes the master codes here (inference_lib/vllm_matgptq.py:177-178);
+                # kept, a layer can be re-sliced to another bitwidth without the checkpoint.
+                layer.matgptq_master = Parameter(qweight.to(layer.matgptq_weights.device), requires_grad=False)
             del layer.qweight
             del layer.scales
 
+    def set_bitwidth(self, layer: torch.nn.Module, bitwidth: int) -> None:
+        """Re-slices a loaded layer to `bitwidth` from its resident master codes (needs
+        `keep_master_codes`).  One device pass over the codes; not for use inside a captured graph
+        (the packed tensor changes size)."""
+        master = getattr(layer, "matgptq_master", None)
+        if master is None:
+            raise RuntimeError("set_bitwidth needs the master codes: load with keep_master_codes")
+        if bitwidth not in (2, 3, 4, 6, 8):
+            raise ValueError("bitwidth must be one of {2, 3, 4, 6, 8}")
+        with torch.no_grad():
+            layer.matgptq_weights = Parameter(self._pack_at(layer, master.data, bitwidth), requires_grad=False)
+            layer.matgptq_bitwidth = bitwidth
+
     def apply(self, layer: torch.nn.Module, x: torch.Tensor,
               bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        bitwidth = getattr(layer, "matgptq_bitwidth", self.bitwidth)
+        if getattr(layer, "matgptq_perm", None) is not None:
+            x = torch.index_select(x, -1, layer.matgptq_perm)
         if getattr(layer, "matgptq_zeros", None) is not None:
             y = torch.ops.matgptq_cuda.matmul_matgptq_zp(
                 x, layer.matgptq_weights, layer.matgptq_scales, layer.matgptq_zeros,
-                self.n_out_features, self.n_in_features, self.bitwidth,
+                self.n_out_features, self.n_in_features, bitwidth,
                 self.config.group_size, self.config.flag)
         else:
             y = torch.ops.matgptq_cuda.matmul_matgptq(
                 x, layer.matgptq_weights, layer.matgptq_scales,
-                self.n_out_features, self.n_in_features, self.bitwidth,
+                self.n_out_features, self.n_in_features, bitwidth,
                 self.config.group_size, self.config.flag)
 
         y = y.view(*x.shape[:-1], y.shape[-1])
