@@ -23,7 +23,7 @@
 extern "C" {
 #endif
 
-#define MATGPTQ_ABI_VERSION 1
+#define MATGPTQ_ABI_VERSION 2
 
 /* error codes */
 #define MATGPTQ_OK 0
@@ -35,6 +35,7 @@ extern "C" {
 #define MATGPTQ_ELAUNCH (-6)   /* the HIP runtime reported an error at launch */
 #define MATGPTQ_EVARIANT (-7)  /* a forced kernel variant does not apply to this problem */
 #define MATGPTQ_ESIZE (-8)     /* a size exceeds what the entry point supports */
+#define MATGPTQ_EWORKSPACE (-9) /* workspace missing or too small */
 
 /* feature_flag bits: the reference's `Features` word
  * (inference_lib/matgptq_cuda/csrc/include/common.cuh:78-86,
@@ -126,6 +127,37 @@ int matgptq_slice_device(const uint8_t *master_dev, int64_t count, int bitwidth,
 int matgptq_dequantize_device(int bitwidth, int group_size, int64_t N, int64_t K,
                               const void *packed_dev, const void *scales_dev,
                               const void *zeros_dev, void *w_dev, void *stream);
+
+/* ---- master-resident codes ------------------------------------------------------
+ * The reference slices the 8-bit master codes once on the host, packs the slice and deletes
+ * the master codes (inference_lib/vllm_matgptq.py:154-178,
+ * inference_lib/inference_demo_transformers.py:30-40): another bitwidth needs the checkpoint
+ * again.  Here the master codes can stay resident as bit planes, most significant first
+ * (N*K/4 words), and the GEMM takes the bitwidth as an argument: it reads the top `bitwidth`
+ * bits of every code plus the bit below them and forms the reference's rounded, saturating
+ * slice (src/quant_utils_matgpqt.py:9-17) in registers.  (bitwidth + 1)/8 bytes per weight
+ * are moved for 2, 3 and 4 bits, one byte for 6 and 8. */
+size_t matgptq_master_words(int64_t N, int64_t K); /* N*K/4, 0 for invalid arguments */
+int matgptq_pack_master_host(const uint8_t *codes_host, int64_t N, int64_t K, uint32_t *planes_host);
+int matgptq_pack_master_device(const uint8_t *codes_dev, int64_t N, int64_t K, uint32_t *planes_dev,
+                               void *stream);
+/* The codes the GEMM sees at `bitwidth`: uint8 [N, K], sliced with the same instruction
+ * sequence the kernels run (bit-exactness checks against matryoshka_slice). */
+int matgptq_unpack_master_host(const uint32_t *planes_host, int64_t N, int64_t K, int bitwidth,
+                               uint8_t *codes_host);
+int matgptq_unpack_master_device(const uint32_t *planes_dev, int64_t N, int64_t K, int bitwidth,
+                                 uint8_t *codes_dev, void *stream);
+/* matgptq_gemm on master-resident planes.  Batch sizes 1..4 at group size 128 (the HBM-bound
+ * regime, where the bytes moved decide) read the planes in the GEMM kernel itself.  Every other
+ * shape slices the planes into the pre-sliced layout first, in `workspace_dev`
+ * (matgptq_gemm_master_workspace_bytes() bytes, 0 when none is needed), and runs the kernel of that
+ * regime on it: two launches, no allocation.  Too small a workspace returns MATGPTQ_EWORKSPACE. */
+size_t matgptq_gemm_master_workspace_bytes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                                           uint32_t flags);
+int matgptq_gemm_master(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                        const void *planes_dev, const void *scales_dev, const void *zeros_dev,
+                        const void *x_dev, void *y_dev, void *workspace_dev, size_t workspace_bytes,
+                        void *stream, uint32_t flags);
 
 /* Human-readable name of the kernel variant matgptq_gemm would launch. */
 int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,

@@ -21,6 +21,9 @@ EXPORTS = (
     "matgptq_pack_host", "matgptq_unpack_host", "matgptq_reorder_scales_host",
     "matgptq_pack_device", "matgptq_unpack_device", "matgptq_reorder_scales_device",
     "matgptq_slice_device", "matgptq_dequantize_device", "matgptq_describe_plan",
+    "matgptq_master_words", "matgptq_pack_master_host", "matgptq_pack_master_device",
+    "matgptq_unpack_master_host", "matgptq_unpack_master_device",
+    "matgptq_gemm_master_workspace_bytes", "matgptq_gemm_master",
 )
 
 _lib = None
@@ -66,6 +69,20 @@ def load() -> ctypes.CDLL:
     L.matgptq_describe_plan.argtypes = [ci, ci, i64, i64, i64, ci, u32, ctypes.c_char_p,
                                         ctypes.c_size_t]
     L.matgptq_describe_plan.restype = ci
+    L.matgptq_master_words.argtypes = [i64, i64]
+    L.matgptq_master_words.restype = ctypes.c_size_t
+    L.matgptq_pack_master_host.argtypes = [vp, i64, i64, vp]
+    L.matgptq_pack_master_host.restype = ci
+    L.matgptq_pack_master_device.argtypes = [vp, i64, i64, vp, vp]
+    L.matgptq_pack_master_device.restype = ci
+    L.matgptq_unpack_master_host.argtypes = [vp, i64, i64, ci, vp]
+    L.matgptq_unpack_master_host.restype = ci
+    L.matgptq_unpack_master_device.argtypes = [vp, i64, i64, ci, vp, vp]
+    L.matgptq_unpack_master_device.restype = ci
+    L.matgptq_gemm_master_workspace_bytes.argtypes = [ci, ci, i64, i64, i64, u32]
+    L.matgptq_gemm_master_workspace_bytes.restype = ctypes.c_size_t
+    L.matgptq_gemm_master.argtypes = [ci, ci, i64, i64, i64, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp, u32]
+    L.matgptq_gemm_master.restype = ci
     _lib = L
     return L
 

@@ -19,8 +19,8 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
                                 bool stream_flavour, size_t smem, hipStream_t);                \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);          \
   hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, hipStream_t);   \
-  hipError_t launch_gemv_b##B(const GemmArgs&, int shape, int W, size_t lds_pad, hipStream_t);  \
-  hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int shape, int W, size_t lds_pad, hipStream_t); \
+  hipError_t launch_gemv_b##B(const GemmArgs&, int shape, int W, size_t lds_pad, bool master, hipStream_t);  \
+  hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int shape, int W, size_t lds_pad, bool master, hipStream_t); \
   hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, hipStream_t); \
   hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
                                        int kc, bool stream_flavour, size_t smem, hipStream_t); \
@@ -35,6 +35,8 @@ MATGPTQ_DECL(8)
 hipError_t launch_pack(const uint8_t*, int64_t, int64_t, int, int, uint32_t*, hipStream_t);
 hipError_t launch_unpack(const uint32_t*, int64_t, int64_t, int, uint8_t*, hipStream_t);
 hipError_t launch_slice(const uint8_t*, int64_t, int, uint8_t*, hipStream_t);
+hipError_t launch_pack_master(const uint8_t*, int64_t, int64_t, uint32_t*, hipStream_t);
+hipError_t launch_master_slice(const uint32_t*, int64_t, int64_t, int, bool, void*, hipStream_t);
 hipError_t launch_reorder(const uint16_t*, int64_t, int64_t, uint16_t*, hipStream_t);
 hipError_t launch_dequant(int, int, int64_t, int64_t, const uint32_t*, const uint16_t*,
                           const uint16_t*, uint16_t*, hipStream_t);
@@ -305,15 +307,18 @@ hipError_t launch_prefill(int bits, bool bf16, const GemmArgs& a, int g, const P
 #undef MATGPTQ_CASE
 }
 
-hipError_t launch_gemv(int bits, bool bf16, const GemmArgs& a, const Plan& p, hipStream_t s) {
+// master: `a.packed` holds master-resident bit planes
+hipError_t launch_gemv(int bits, bool bf16, const GemmArgs& a, const Plan& p, bool master, hipStream_t s) {
 #define MATGPTQ_CASE(B) \
-  case B: return bf16 ? launch_gemv_b##B##_bf16(a, p.shape, p.W, p.pad, s) : launch_gemv_b##B(a, p.shape, p.W, p.pad, s);
+  case B: return bf16 ? launch_gemv_b##B##_bf16(a, p.shape, p.W, p.pad, master, s) \
+                      : launch_gemv_b##B(a, p.shape, p.W, p.pad, master, s);
   switch (bits) {
     MATGPTQ_CASE(2)
     MATGPTQ_CASE(3)
     MATGPTQ_CASE(4)
     MATGPTQ_CASE(6)
-    default: return bf16 ? launch_gemv_b8_bf16(a, p.shape, p.W, p.pad, s) : launch_gemv_b8(a, p.shape, p.W, p.pad, s);
+    default: return bf16 ? launch_gemv_b8_bf16(a, p.shape, p.W, p.pad, master, s)
+                         : launch_gemv_b8(a, p.shape, p.W, p.pad, master, s);
   }
 #undef MATGPTQ_CASE
 }
@@ -351,22 +356,26 @@ const char* matgptq_strerror(int code) {
     case MATGPTQ_ELAUNCH: return "HIP launch failed";
     case MATGPTQ_EVARIANT: return "forced kernel variant does not apply to this problem";
     case MATGPTQ_ESIZE: return "size exceeds the supported maximum";
+    case MATGPTQ_EWORKSPACE: return "workspace missing or smaller than matgptq_gemm_master_workspace_bytes()";
     default: return "unknown error";
   }
 }
 
-int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
-                 const void* packed_dev, const void* scales_dev, const void* zeros_dev,
-                 const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
+// checks, plan, launch; `master_planes`: the weight operand is master-resident bit planes and
+// the plan must be the gemv kernel (the caller has made sure of it)
+static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M, const void* weights_dev,
+                    const void* scales_dev, const void* zeros_dev, const void* x_dev, void* y_dev,
+                    void* stream, uint32_t flags, bool master_planes) {
   if (int e = check_problem(bitwidth, group_size, N, K)) return e;
   if (M <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return MATGPTQ_ESIZE;
-  // the kernels address the packed tensor with 32-bit byte offsets
-  if ((uint64_t)N * (uint64_t)K / 8 * (uint64_t)bitwidth >= (1ull << 32)) return MATGPTQ_ESIZE;
-  if (!packed_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
+  // the kernels address the weight tensor with 32-bit byte offsets
+  if ((uint64_t)N * (uint64_t)K / 8 * (uint64_t)(master_planes ? 8 : bitwidth) >= (1ull << 32)) return MATGPTQ_ESIZE;
+  if (!weights_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &p)) return e;
+  if (master_planes && !(p.gemv && (p.shape == 1 || p.shape == 2))) return MATGPTQ_EVARIANT;
   GemmArgs a;
-  a.packed = static_cast<const uint32_t*>(packed_dev);
+  a.packed = static_cast<const uint32_t*>(weights_dev);
   a.scales = static_cast<const uint16_t*>(scales_dev);
   a.zeros = static_cast<const uint16_t*>(zeros_dev);
   a.x = static_cast<const uint16_t*>(x_dev);
@@ -379,7 +388,7 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
   a.row_blocks = (int)(N / 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
-  const hipError_t err = p.gemv     ? launch_gemv(bitwidth, bf16, a, p, s)
+  const hipError_t err = p.gemv     ? launch_gemv(bitwidth, bf16, a, p, master_planes, s)
                          : p.decode ? launch_decode(bitwidth, bf16, a, group_size, p, s)
                          : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, s)
                                     : launch_prefill(bitwidth, bf16, a, group_size, p, s);
@@ -388,6 +397,76 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
     if (hipStreamSynchronize(s) != hipSuccess) return MATGPTQ_ELAUNCH;
   }
   return MATGPTQ_OK;
+}
+
+int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                 const void* packed_dev, const void* scales_dev, const void* zeros_dev,
+                 const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
+  return run_gemm(bitwidth, group_size, N, K, M, packed_dev, scales_dev, zeros_dev, x_dev, y_dev, stream,
+                  flags, false);
+}
+
+// does the GEMM at this shape read the planes itself (gemv kernel), or does it need the
+// pre-sliced tensor in a workspace first?
+static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M, bool zp,
+                               uint32_t flags, bool* direct) {
+  if (int e = check_problem(bitwidth, group_size, N, K)) return e;
+  if (M <= 0) return MATGPTQ_ESIZE;
+  Plan p;
+  if (int e = make_plan(bitwidth, group_size, N, K, M, zp, flags, &p)) return e;
+  *direct = p.gemv && (p.shape == 1 || p.shape == 2);
+  return MATGPTQ_OK;
+}
+
+size_t matgptq_gemm_master_workspace_bytes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                                           uint32_t flags) {
+  bool direct = false;
+  if (master_reads_planes(bitwidth, group_size, N, K, M, true, flags, &direct) != MATGPTQ_OK) return 0;
+  return direct ? 0 : matgptq_packed_words(bitwidth, N, K) * 4;
+}
+
+static int gemm_master_impl(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                            const void* planes_dev, const void* scales_dev, const void* zeros_dev,
+                            const void* x_dev, void* y_dev, void* workspace_dev, size_t workspace_bytes,
+                            void* stream, uint32_t flags) {
+  bool direct = false;
+  if (int e = master_reads_planes(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &direct)) return e;
+  if (!planes_dev) return MATGPTQ_ENULL;
+  if (direct)
+    return run_gemm(bitwidth, group_size, N, K, M, planes_dev, scales_dev, zeros_dev, x_dev, y_dev, stream,
+                    flags, true);
+  // two launches: slice the planes into the pre-sliced layout, then the GEMM of that regime
+  const size_t need = matgptq_packed_words(bitwidth, N, K) * 4;
+  if (!workspace_dev || workspace_bytes < need) return MATGPTQ_EWORKSPACE;
+  if (launch_master_slice(static_cast<const uint32_t*>(planes_dev), N, K, bitwidth, true, workspace_dev,
+                          static_cast<hipStream_t>(stream)) != hipSuccess)
+    return MATGPTQ_ELAUNCH;
+  return run_gemm(bitwidth, group_size, N, K, M, workspace_dev, scales_dev, zeros_dev, x_dev, y_dev, stream,
+                  flags, false);
+}
+
+int matgptq_gemm_master(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                        const void* planes_dev, const void* scales_dev, const void* zeros_dev,
+                        const void* x_dev, void* y_dev, void* workspace_dev, size_t workspace_bytes,
+                        void* stream, uint32_t flags) {
+  return gemm_master_impl(bitwidth, group_size, N, K, M, planes_dev, scales_dev, zeros_dev, x_dev, y_dev,
+                          workspace_dev, workspace_bytes, stream, flags);
+}
+
+int matgptq_pack_master_device(const uint8_t* codes_dev, int64_t N, int64_t K, uint32_t* planes_dev,
+                               void* stream) {
+  if (int e = check_problem(8, -1, N, K)) return e;
+  if (!codes_dev || !planes_dev) return MATGPTQ_ENULL;
+  return launch_pack_master(codes_dev, N, K, planes_dev, static_cast<hipStream_t>(stream)) == hipSuccess
+             ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+int matgptq_unpack_master_device(const uint32_t* planes_dev, int64_t N, int64_t K, int bitwidth,
+                                 uint8_t* codes_dev, void* stream) {
+  if (int e = check_problem(bitwidth, -1, N, K)) return e;
+  if (!planes_dev || !codes_dev) return MATGPTQ_ENULL;
+  return launch_master_slice(planes_dev, N, K, bitwidth, false, codes_dev, static_cast<hipStream_t>(stream)) ==
+                 hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
 }
 
 int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,

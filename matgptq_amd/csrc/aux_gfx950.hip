@@ -3,6 +3,7 @@
 // (inference_lib/matgptq_cuda/csrc/bindings.cpp:63-83,99-141) and give tests a
 // device-side view of the packed codes.  All are byte/integer work, HBM-bound.
 #include "device_common.h"
+#include "master_layout.h"
 
 namespace matgptq {
 
@@ -141,6 +142,78 @@ dequant_kernel(const uint32_t* __restrict__ packed, const uint16_t* __restrict__
   emit(std::integral_constant<int, 3>{});
 }
 
+// ---- master-resident bit planes (master_layout.h) --------------------------------------
+// 32 codes of a lane slot from row-major uint8 [N, K]
+__device__ __forceinline__ void read_lane_codes(const uint8_t* __restrict__ row, uint8_t (&c)[32]) {
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const uint2 v = *reinterpret_cast<const uint2*>(row + j * 32);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      c[j * 8 + e] = (uint8_t)(v.x >> (8 * e));
+      c[j * 8 + 4 + e] = (uint8_t)(v.y >> (8 * e));
+    }
+  }
+}
+
+// master codes [N, K] -> bit planes; one thread = one lane slot of one tile
+__global__ void __launch_bounds__(256)
+pack_master_kernel(const uint8_t* __restrict__ codes, uint32_t* __restrict__ out, int k_tiles,
+                   int64_t K, int64_t total_slots) {
+  const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot >= total_slots) return;
+  const int lane = (int)(slot & 63);
+  const int64_t tile = slot >> 6;
+  const int64_t rb = tile / k_tiles, kb = tile - rb * k_tiles;
+  uint8_t c[32];
+  read_lane_codes(codes + (rb * 16 + (lane & 15)) * K + kb * 128 + (lane >> 4) * 8, c);
+  uint32_t w[8];
+  master_encode_lane(c, w);
+  uint32_t* t = out + tile * kMasterTileWords;
+#pragma unroll
+  for (int i = 0; i < 8; i++) t[master_word_offset(lane, i)] = w[i];
+}
+
+// bit planes -> codes sliced to BITS with the sequence the GEMM kernels run:
+// SLICED_PACKED false: uint8 [N, K] (bit-exactness checks);
+// SLICED_PACKED true : the pre-sliced tile layout of layout.h (input of the kernels that do not
+//                      read the planes themselves)
+template <int BITS, bool SLICED_PACKED>
+__global__ void __launch_bounds__(256)
+master_slice_kernel(const uint32_t* __restrict__ planes, void* __restrict__ out, int k_tiles,
+                    int64_t K, int64_t total_slots) {
+  const int64_t slot = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (slot >= total_slots) return;
+  const int lane = (int)(slot & 63);
+  const int64_t tile = slot >> 6;
+  const int64_t rb = tile / k_tiles, kb = tile - rb * k_tiles;
+  const uint32_t* t = planes + tile * kMasterTileWords;
+  uint32_t w[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) w[i] = i < master_words(BITS) ? t[master_word_offset(lane, i)] : 0u;
+  uint8_t c[32];
+  master_decode_lane<BITS>(w, c);
+  if constexpr (SLICED_PACKED) {
+    uint32_t pw[BITS];
+    Codec<BITS>::encode_lane(c, pw);
+    uint32_t* o = static_cast<uint32_t*>(out) + tile * tile_words(BITS);
+#pragma unroll
+    for (int i = 0; i < BITS; i++) o[word_offset(BITS, lane, i)] = pw[i];
+  } else {
+    uint8_t* row = static_cast<uint8_t*>(out) + (rb * 16 + (lane & 15)) * K + kb * 128 + (lane >> 4) * 8;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        lo |= (uint32_t)c[j * 8 + e] << (8 * e);
+        hi |= (uint32_t)c[j * 8 + 4 + e] << (8 * e);
+      }
+      *reinterpret_cast<uint2*>(row + j * 32) = make_uint2(lo, hi);
+    }
+  }
+}
+
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
 }  // namespace
@@ -172,6 +245,38 @@ hipError_t launch_unpack(const uint32_t* packed, int64_t N, int64_t K, int bits,
     case 6: hipLaunchKernelGGL(unpack_kernel<6>, grid, block, 0, s, packed, codes, k_tiles, K, slots); break;
     default: hipLaunchKernelGGL(unpack_kernel<8>, grid, block, 0, s, packed, codes, k_tiles, K, slots); break;
   }
+  return hipGetLastError();
+}
+
+hipError_t launch_pack_master(const uint8_t* codes, int64_t N, int64_t K, uint32_t* out, hipStream_t s) {
+  const int k_tiles = (int)(K / 128);
+  const int64_t slots = (N / 16) * (int64_t)k_tiles * 64;
+  hipLaunchKernelGGL(pack_master_kernel, dim3(blocks_for(slots, 256)), dim3(256), 0, s, codes, out, k_tiles, K, slots);
+  return hipGetLastError();
+}
+
+// sliced_packed: write the pre-sliced tile layout instead of uint8 [N, K]
+hipError_t launch_master_slice(const uint32_t* planes, int64_t N, int64_t K, int bits, bool sliced_packed,
+                               void* out, hipStream_t s) {
+  const int k_tiles = (int)(K / 128);
+  const int64_t slots = (N / 16) * (int64_t)k_tiles * 64;
+  const dim3 grid(blocks_for(slots, 256)), block(256);
+#define MATGPTQ_MS(B)                                                                                         \
+  case B:                                                                                                     \
+    if (sliced_packed) hipLaunchKernelGGL((master_slice_kernel<B, true>), grid, block, 0, s, planes, out, k_tiles, K, slots); \
+    else hipLaunchKernelGGL((master_slice_kernel<B, false>), grid, block, 0, s, planes, out, k_tiles, K, slots);  \
+    break;
+  switch (bits) {
+    MATGPTQ_MS(2)
+    MATGPTQ_MS(3)
+    MATGPTQ_MS(4)
+    MATGPTQ_MS(6)
+    default:
+      if (sliced_packed) hipLaunchKernelGGL((master_slice_kernel<8, true>), grid, block, 0, s, planes, out, k_tiles, K, slots);
+      else hipLaunchKernelGGL((master_slice_kernel<8, false>), grid, block, 0, s, planes, out, k_tiles, K, slots);
+      break;
+  }
+#undef MATGPTQ_MS
   return hipGetLastError();
 }
 

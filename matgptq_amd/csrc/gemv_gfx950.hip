@@ -24,7 +24,7 @@
 //     acc += scale * (D - off - zero / 2^(8-b) * xs)
 // which is  sum_k scale ((c << (8-b)) - zero) x / 2^(8-b)  over the group.  The partial sums
 // of the four lane quarters and the W waves meet in LDS once, at the end.
-#include "device_common.h"
+#include "tile_format.h"
 
 #ifndef MATGPTQ_BITS
 #error "compile with -DMATGPTQ_BITS={2,3,4,6,8}"
@@ -56,8 +56,11 @@ __device__ __forceinline__ float row_sum16(float v) {
 // LDS bytes per wave: X' of one round for MB batch rows + a block of zeros
 constexpr int gemv_wave_lds(int t, int mb) { return mb * t * 256 + 256; }
 
-template <int BITS, bool ZP, int T, int R, int MB>
+// MASTER: `a.packed` holds master-resident bit planes (master_layout.h); the rounded slice to
+// BITS is formed in registers while the raw pairs are built.
+template <int BITS, bool ZP, int T, int R, int MB, bool MASTER>
 __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
+  using Fmt = TileFormat<BITS, MASTER>;
   constexpr int TH = (T + 3) / 4;  // groups of four tiles per round
   constexpr float kMul = (float)(1 << (8 - BITS));
   constexpr int kXBytes = MB * T * 256;
@@ -75,8 +78,8 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
   float* red = reinterpret_cast<float*>(smem + W * kWaveBytes);   // [W][R * MB][64]
   if (lane < 16) *reinterpret_cast<uint4*>(xw + kXBytes + lane * 16) = make_uint4(0, 0, 0, 0);
 
-  constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
-  const UnpackConsts<BITS> consts;
+  constexpr uint32_t tile_bytes = Fmt::kTileBytes;
+  const typename Fmt::Consts consts;
   // activation operand: row n of A is batch row n % 4 while tile u = n / 4 of a group of four is
   // multiplied; the batch rows beyond M repeat row M - 1 (their results are never stored)
   const int arow = (n & 3) < a.M ? (n & 3) : a.M - 1;
@@ -106,7 +109,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         xv[m][h] = __builtin_amdgcn_raw_buffer_load_b128(xr, lane * 16, (uint32_t)(kt0 + 4 * h) * 256u, 0);
     }
     uint16_t sv[R][TH], zv[R][TH];
-    uint32_t w[R][T][BITS];
+    uint32_t w[R][T][Fmt::kWords];
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
       const bool rows = rb0 + rr < a.row_blocks;
@@ -125,7 +128,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
       const uint32_t g0 = (uint32_t)(rb0 + rr) * a.k_tiles + kt0;
       const BufRsrc wr = make_rsrc(a.packed, rows ? (g0 + nt) * tile_bytes : 0u);
 #pragma unroll
-      for (int i = 0; i < T; i++) load_tile_words<BITS>(wr, (g0 + i) * tile_bytes, lane, w[rr][i]);
+      for (int i = 0; i < T; i++) Fmt::load(wr, (g0 + i) * tile_bytes, lane, w[rr][i]);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -144,13 +147,13 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         sx = dot2(v.p[1], ones, sx);
         sx = dot2(v.p[2], ones, sx);
         sx = dot2(v.p[3], ones, sx);
-        if constexpr (BITS != 8) {
-          // pair i of octet j is scaled by 2^-p(j, i); only 2-bit codes depend on j (its parity)
-          const bool odd = BITS == 2 && (n & 4) != 0;  // octet = chunk / 4, chunk = lane % 16
-          const float i0 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 0)), i1 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 1));
-          const float i2 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 2)), i3 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(0, 3));
-          const float o0 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 0)), o1 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 1));
-          const float o2 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 2)), o3 = 1.0f / (float)(1 << Codec<BITS>::raw_shift(1, 3));
+        if constexpr (Fmt::kScaledX) {
+          // pair i of octet j is scaled by 2^-p(j, i); only pre-sliced 2-bit codes depend on j (its parity)
+          const bool odd = BITS == 2 && !MASTER && (n & 4) != 0;  // octet = chunk / 4, chunk = lane % 16
+          const float i0 = 1.0f / (float)(1 << Fmt::raw_shift(0, 0)), i1 = 1.0f / (float)(1 << Fmt::raw_shift(0, 1));
+          const float i2 = 1.0f / (float)(1 << Fmt::raw_shift(0, 2)), i3 = 1.0f / (float)(1 << Fmt::raw_shift(0, 3));
+          const float o0 = 1.0f / (float)(1 << Fmt::raw_shift(1, 0)), o1 = 1.0f / (float)(1 << Fmt::raw_shift(1, 1));
+          const float o2 = 1.0f / (float)(1 << Fmt::raw_shift(1, 2)), o3 = 1.0f / (float)(1 << Fmt::raw_shift(1, 3));
           v.p[0] = v.p[0] * h2_splat(odd ? o0 : i0);
           v.p[1] = v.p[1] * h2_splat(odd ? o1 : i1);
           v.p[2] = v.p[2] * h2_splat(odd ? o2 : i2);
@@ -181,13 +184,13 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 #pragma unroll
       for (int rr = 0; rr < R; rr++) {
         Frag bw;
-        raw_octet<BITS, 0>(w[rr][i], consts, bw.u);
+        Fmt::template raw<0>(w[rr][i], consts, bw.u);
         d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[0].h, bw.h, d[rr], 0, 0, 0);
-        raw_octet<BITS, 1>(w[rr][i], consts, bw.u);
+        Fmt::template raw<1>(w[rr][i], consts, bw.u);
         d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[1].h, bw.h, d[rr], 0, 0, 0);
-        raw_octet<BITS, 2>(w[rr][i], consts, bw.u);
+        Fmt::template raw<2>(w[rr][i], consts, bw.u);
         d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[2].h, bw.h, d[rr], 0, 0, 0);
-        raw_octet<BITS, 3>(w[rr][i], consts, bw.u);
+        Fmt::template raw<3>(w[rr][i], consts, bw.u);
         d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[3].h, bw.h, d[rr], 0, 0, 0);
       }
       if (u == 3 || i == T - 1) {
@@ -223,12 +226,12 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 }
 
 // WPE: waves per SIMD the register allocation is held to
-template <int BITS, bool ZP, int T, int R, int MB, int WPE>
+template <int BITS, bool ZP, int T, int R, int MB, int WPE, bool MASTER>
 __global__ void __launch_bounds__(1024, WPE) gemv_kernel(const GemmArgs a, const int W) {
-  gemv_body<BITS, ZP, T, R, MB>(a, W);
+  gemv_body<BITS, ZP, T, R, MB, MASTER>(a, W);
 }
 
-template <bool ZP, int T, int R, int MB, int WPE>
+template <bool ZP, int T, int R, int MB, int WPE, bool MASTER>
 hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stream) {
   const dim3 grid((a.row_blocks + R - 1) / R), block(64 * W);
   size_t smem = (size_t)W * gemv_wave_lds(T, MB) + (size_t)W * R * MB * 256;
@@ -238,34 +241,52 @@ hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stre
     // more than 64 KiB of dynamic LDS has to be allowed once per kernel
     static bool allowed = false;
     if (!allowed) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, T, R, MB, WPE>),
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, T, R, MB, WPE, MASTER>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
       allowed = true;
     }
   }
-  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, T, R, MB, WPE>), grid, block, smem, stream, a, W);
+  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, T, R, MB, WPE, MASTER>), grid, block, smem, stream, a, W);
   return hipGetLastError();
 }
 
-// shapes built: (T tiles per wave and round, R row blocks per workgroup)
-template <bool ZP, int MB>
+// shapes built: (T tiles per wave and round, R row blocks per workgroup); the master-resident
+// storage takes the two shapes the planner uses
+template <bool ZP, int MB, bool MASTER>
 hipError_t launch_shape(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t s) {
-  switch (shape) {
-    case 0: return launch_one<ZP, 8, 1, MB, 4>(a, W, lds_pad, s);
-    case 1: return launch_one<ZP, 4, 1, MB, 4>(a, W, lds_pad, s);
-    case 2: return launch_one<ZP, 4, 2, MB, 4>(a, W, lds_pad, s);
-    case 3: return launch_one<ZP, 2, 2, MB, 4>(a, W, lds_pad, s);
-    case 4: return launch_one<ZP, 2, 4, MB, 4>(a, W, lds_pad, s);
-    default: return launch_one<ZP, 2, 1, MB, 4>(a, W, lds_pad, s);
+  if constexpr (MASTER) {
+    if (shape == 2) return launch_one<ZP, 4, 2, MB, 4, true>(a, W, lds_pad, s);
+    if (shape == 1) return launch_one<ZP, 4, 1, MB, 4, true>(a, W, lds_pad, s);
+    return hipErrorInvalidValue;
+  } else {
+    switch (shape) {
+      case 0: return launch_one<ZP, 8, 1, MB, 4, false>(a, W, lds_pad, s);
+      case 1: return launch_one<ZP, 4, 1, MB, 4, false>(a, W, lds_pad, s);
+      case 2: return launch_one<ZP, 4, 2, MB, 4, false>(a, W, lds_pad, s);
+      case 3: return launch_one<ZP, 2, 2, MB, 4, false>(a, W, lds_pad, s);
+      case 4: return launch_one<ZP, 2, 4, MB, 4, false>(a, W, lds_pad, s);
+      default: return launch_one<ZP, 2, 1, MB, 4, false>(a, W, lds_pad, s);
+    }
   }
+}
+
+template <bool MASTER>
+hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t stream) {
+  const bool zp = a.zeros != nullptr;
+  if (a.M == 1)
+    return zp ? launch_shape<true, 1, MASTER>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, 1, MASTER>(a, shape, W, lds_pad, stream);
+  return zp ? launch_shape<true, 4, MASTER>(a, shape, W, lds_pad, stream)
+            : launch_shape<false, 4, MASTER>(a, shape, W, lds_pad, stream);
 }
 
 }  // namespace
 
 // Entry of this translation unit.  shape: index into the (T, R) table above; W: waves per
 // workgroup (1..16); lds_pad: dynamic LDS to ask for when it exceeds what the kernel needs
-// (limits how many workgroups share a CU).  Group size 128 and M <= 4 only.
+// (limits how many workgroups share a CU); master: `a.packed` holds master-resident bit planes
+// (shapes 1 and 2 only).  Group size 128 and M <= 4 only.
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 #if MATGPTQ_BF16
@@ -273,13 +294,10 @@ hipError_t launch_shape(const GemmArgs& a, int shape, int W, size_t lds_pad, hip
 #else
 #define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_gemv_b, MATGPTQ_BITS)
 #endif
-hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t stream) {
-  const bool zp = a.zeros != nullptr;
-  if (a.M == 1)
-    return zp ? launch_shape<true, 1>(a, shape, W, lds_pad, stream)
-              : launch_shape<false, 1>(a, shape, W, lds_pad, stream);
-  return zp ? launch_shape<true, 4>(a, shape, W, lds_pad, stream)
-            : launch_shape<false, 4>(a, shape, W, lds_pad, stream);
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int shape, int W, size_t lds_pad, bool master,
+                               hipStream_t stream) {
+  return master ? launch_storage<true>(a, shape, W, lds_pad, stream)
+                : launch_storage<false>(a, shape, W, lds_pad, stream);
 }
 
 }  // namespace matgptq

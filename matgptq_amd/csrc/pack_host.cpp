@@ -6,6 +6,7 @@
 
 #include "../../include/matgptq_abi.h"
 #include "layout.h"
+#include "master_layout.h"
 
 namespace matgptq {
 
@@ -63,6 +64,26 @@ static void unpack_impl(const uint32_t* packed, int64_t N, int64_t K, uint8_t* c
   }
 }
 
+template <int BITS>
+static void master_slice_impl(const uint32_t* planes, int64_t N, int64_t K, uint8_t* codes) {
+  const int64_t row_blocks = N / kTileRows, k_blocks = K / kTileCols;
+#pragma omp parallel for schedule(static)
+  for (int64_t rb = 0; rb < row_blocks; rb++) {
+    for (int64_t kb = 0; kb < k_blocks; kb++) {
+      const uint32_t* tile = planes + (rb * k_blocks + kb) * kMasterTileWords;
+      for (int lane = 0; lane < kLanes; lane++) {
+        uint32_t w[8];
+        for (int i = 0; i < 8; i++) w[i] = i < master_words(BITS) ? tile[master_word_offset(lane, i)] : 0u;
+        uint8_t c[32];
+        master_decode_lane<BITS>(w, c);
+        uint8_t* row = codes + (rb * kTileRows + lane % 16) * K + kb * kTileCols + (lane / 16) * 8;
+        for (int j = 0; j < 4; j++)
+          for (int e = 0; e < 8; e++) row[j * 32 + e] = c[j * 8 + e];
+      }
+    }
+  }
+}
+
 }  // namespace matgptq
 
 using namespace matgptq;
@@ -99,6 +120,46 @@ int matgptq_unpack_host(const uint32_t* packed_host, int64_t N, int64_t K, int b
     case 4: unpack_impl<4>(packed_host, N, K, codes_host); break;
     case 6: unpack_impl<6>(packed_host, N, K, codes_host); break;
     case 8: unpack_impl<8>(packed_host, N, K, codes_host); break;
+  }
+  return MATGPTQ_OK;
+}
+
+size_t matgptq_master_words(int64_t N, int64_t K) {
+  if (N <= 0 || K <= 0 || N % kTileRows != 0 || K % kTileCols != 0) return 0;
+  return (size_t)N * (size_t)K / 4;
+}
+
+int matgptq_pack_master_host(const uint8_t* codes_host, int64_t N, int64_t K, uint32_t* out_host) {
+  if (int e = check_problem(8, -1, N, K)) return e;
+  if (!codes_host || !out_host) return MATGPTQ_ENULL;
+  const int64_t row_blocks = N / kTileRows, k_blocks = K / kTileCols;
+#pragma omp parallel for schedule(static)
+  for (int64_t rb = 0; rb < row_blocks; rb++)
+    for (int64_t kb = 0; kb < k_blocks; kb++) {
+      uint32_t* tile = out_host + (rb * k_blocks + kb) * kMasterTileWords;
+      for (int lane = 0; lane < kLanes; lane++) {
+        const uint8_t* row = codes_host + (rb * kTileRows + lane % 16) * K + kb * kTileCols + (lane / 16) * 8;
+        uint8_t c[32];
+        for (int j = 0; j < 4; j++)
+          for (int e = 0; e < 8; e++) c[j * 8 + e] = row[j * 32 + e];
+        uint32_t w[8];
+        master_encode_lane(c, w);
+        for (int i = 0; i < 8; i++) tile[master_word_offset(lane, i)] = w[i];
+      }
+    }
+  return MATGPTQ_OK;
+}
+
+int matgptq_unpack_master_host(const uint32_t* planes_host, int64_t N, int64_t K, int bitwidth,
+                               uint8_t* codes_host) {
+  if (int e = check_problem(bitwidth, -1, N, K)) return e;
+  if (!planes_host || !codes_host) return MATGPTQ_ENULL;
+  switch (bitwidth) {
+    case 2: master_slice_impl<2>(planes_host, N, K, codes_host); break;
+    case 3: master_slice_impl<3>(planes_host, N, K, codes_host); break;
+    case 4: master_slice_impl<4>(planes_host, N, K, codes_host); break;
+    case 6: master_slice_impl<6>(planes_host, N, K, codes_host); break;
+    case 8: master_slice_impl<8>(planes_host, N, K, codes_host); break;
   }
   return MATGPTQ_OK;
 }

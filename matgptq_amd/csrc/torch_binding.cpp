@@ -128,10 +128,11 @@ Tensor reorder_matgptq_scales(const Tensor& scales, int64_t n_out_features, int6
 }
 
 // matmul_matgptq (bindings.cpp:146-191) and its zero-point extension.
+// `master`: `weights` are master-resident bit planes (N*K/4 words) instead of a pre-sliced tensor
 Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& scales,
                    const c10::optional<Tensor>& zeros, int64_t n_out_features,
                    int64_t n_in_features, int64_t bitwidth, int64_t group_size,
-                   int64_t feature_flag) {
+                   int64_t feature_flag, bool master = false) {
   TORCH_CHECK(input.is_cuda() && weights.is_cuda() && scales.is_cuda(),
               "matmul_matgptq: input, matgptq_weights and matgptq_scales must be GPU tensors");
   TORCH_CHECK(input.device() == weights.device() && input.device() == scales.device(),
@@ -141,7 +142,7 @@ Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& sca
   TORCH_CHECK(weights.dim() == 1, "qweights must be 1D");
   check_bits_group(bitwidth, group_size, n_in_features);
   check_tiling(n_out_features, n_in_features);
-  TORCH_CHECK(weights.size(0) == bitwidth * n_out_features * n_in_features / 32,
+  TORCH_CHECK(weights.size(0) == (master ? 8 : bitwidth) * n_out_features * n_in_features / 32,
               "matgptq_weights has the wrong size");
   const bool bf16 = (feature_flag & MATGPTQ_FLAG_BF16) != 0;
   // the reference trusts the flag (bindings.cpp:171-174); a mismatch is reported here
@@ -175,9 +176,23 @@ Tensor matmul_impl(const Tensor& input, const Tensor& weights, const Tensor& sca
   Tensor out = torch::empty({m, n_out_features}, input.options());
   if (m == 0) return out;
   const uint32_t flags = (uint32_t)feature_flag | MATGPTQ_FLAG_ASYNC;
-  const int code = matgptq_gemm((int)bitwidth, (int)group_size, n_out_features, n_in_features, m,
-                                weights.data_ptr(), scales.data_ptr(), zeros_ptr, input_c.data_ptr(),
-                                out.data_ptr(), stream_of(dev), flags);
+  int code;
+  if (master) {
+    // shapes outside the kernel that reads the planes itself need the pre-sliced tensor in a
+    // workspace: taken from torch's caching allocator (capturable like the output)
+    const size_t ws_bytes = matgptq_gemm_master_workspace_bytes((int)bitwidth, (int)group_size, n_out_features,
+                                                               n_in_features, m, flags);
+    Tensor ws;
+    if (ws_bytes > 0) ws = torch::empty({(int64_t)ws_bytes}, input.options().dtype(torch::kUInt8));
+    code = matgptq_gemm_master((int)bitwidth, (int)group_size, n_out_features, n_in_features, m,
+                               weights.data_ptr(), scales.data_ptr(), zeros_ptr, input_c.data_ptr(),
+                               out.data_ptr(), ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes,
+                               stream_of(dev), flags);
+  } else {
+    code = matgptq_gemm((int)bitwidth, (int)group_size, n_out_features, n_in_features, m,
+                        weights.data_ptr(), scales.data_ptr(), zeros_ptr, input_c.data_ptr(),
+                        out.data_ptr(), stream_of(dev), flags);
+  }
   check_abi(code, "matmul_matgptq");
   if (!(feature_flag & MATGPTQ_FLAG_ASYNC)) {
     // SYNC mode of the reference: the call returns after the kernel (matgptq_gemm.cu:1060-1062)
@@ -198,6 +213,60 @@ Tensor matmul_matgptq_zp(const Tensor& input, const Tensor& weights, const Tenso
                          int64_t bitwidth, int64_t group_size, int64_t feature_flag) {
   return matmul_impl(input, weights, scales, zeros, n_out_features, n_in_features, bitwidth,
                      group_size, feature_flag);
+}
+
+// ---- master-resident codes (additive; see include/matgptq_abi.h) ----
+Tensor matmul_matgptq_master(const Tensor& input, const Tensor& planes, const Tensor& scales,
+                             const c10::optional<Tensor>& zeros, int64_t n_out_features,
+                             int64_t n_in_features, int64_t bitwidth, int64_t group_size,
+                             int64_t feature_flag) {
+  return matmul_impl(input, planes, scales, zeros, n_out_features, n_in_features, bitwidth, group_size,
+                     feature_flag, true);
+}
+
+Tensor pack_matgptq_master_resident(const Tensor& qweights) {
+  TORCH_CHECK(qweights.dtype() == torch::kUInt8, "qweights must be uint8");
+  TORCH_CHECK(qweights.is_contiguous(), "qweights must be contiguous");
+  TORCH_CHECK(qweights.dim() == 2, "qweights must be 2D (n_out_features, n_in_features)");
+  const int64_t n = qweights.size(0), k = qweights.size(1);
+  check_tiling(n, k);
+  const at::Device dev = target_device(qweights);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+  const int64_t words = n * k / 4;
+  Tensor out = torch::empty({words}, torch::dtype(torch::kUInt32).device(dev));
+  if (qweights.is_cuda()) {
+    check_abi(matgptq_pack_master_device(qweights.data_ptr<uint8_t>(), n, k, static_cast<uint32_t*>(out.data_ptr()),
+                                         stream_of(dev)),
+              "pack_matgptq_master_resident");
+  } else {
+    Tensor host = torch::empty({words}, torch::dtype(torch::kUInt32).device(torch::kCPU));
+    check_abi(matgptq_pack_master_host(qweights.data_ptr<uint8_t>(), n, k, static_cast<uint32_t*>(host.data_ptr())),
+              "pack_matgptq_master_resident");
+    out.copy_(host);
+  }
+  return out;
+}
+
+Tensor unpack_matgptq_master_resident(const Tensor& planes, int64_t n_out_features, int64_t n_in_features,
+                                      int64_t bitwidth) {
+  TORCH_CHECK(planes.dtype() == torch::kUInt32 && planes.dim() == 1 && planes.is_contiguous(),
+              "master planes must be a contiguous 1D uint32 tensor");
+  check_bits_group(bitwidth, -1, n_in_features);
+  check_tiling(n_out_features, n_in_features);
+  TORCH_CHECK(planes.size(0) == n_out_features * n_in_features / 4, "master planes have the wrong size");
+  Tensor out = torch::empty({n_out_features, n_in_features}, planes.options().dtype(torch::kUInt8));
+  if (planes.is_cuda()) {
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(planes.device());
+    check_abi(matgptq_unpack_master_device(static_cast<const uint32_t*>(planes.data_ptr()), n_out_features,
+                                           n_in_features, (int)bitwidth, out.data_ptr<uint8_t>(),
+                                           stream_of(planes.device())),
+              "unpack_matgptq_master_resident");
+  } else {
+    check_abi(matgptq_unpack_master_host(static_cast<const uint32_t*>(planes.data_ptr()), n_out_features,
+                                         n_in_features, (int)bitwidth, out.data_ptr<uint8_t>()),
+              "unpack_matgptq_master_resident");
+  }
+  return out;
 }
 
 // Debug / test helpers: the codes and the dense weight a packed tensor stands for.
@@ -303,6 +372,11 @@ TORCH_LIBRARY(matgptq_cuda, m) {
   m.def("unpack_matgptq_qweights(Tensor matgptq_weights, int n_out_features, int n_in_features, "
         "int bitwidth) -> Tensor");
   m.def("slice_matgptq_master(Tensor master, int bitwidth) -> Tensor");
+  m.def("pack_matgptq_master_resident(Tensor qweights) -> Tensor");
+  m.def("unpack_matgptq_master_resident(Tensor planes, int n_out_features, int n_in_features, "
+        "int bitwidth) -> Tensor");
+  m.def("matmul_matgptq_master(Tensor input, Tensor planes, Tensor matgptq_scales, Tensor? matgptq_zeros, "
+        "int n_out_features, int n_in_features, int bitwidth, int group_size, int feature_flag) -> Tensor");
   m.def("dequantize_matgptq(Tensor matgptq_weights, Tensor matgptq_scales, Tensor? matgptq_zeros, "
         "int n_out_features, int n_in_features, int bitwidth, int group_size) -> Tensor");
 }
@@ -315,12 +389,15 @@ TORCH_LIBRARY_IMPL(matgptq_cuda, CompositeExplicitAutograd, m) {
   m.impl("pack_matgptq_master", TORCH_FN(pack_matgptq_master));
   m.impl("reorder_matgptq_scales", TORCH_FN(reorder_matgptq_scales));
   m.impl("unpack_matgptq_qweights", TORCH_FN(unpack_matgptq_qweights));
+  m.impl("pack_matgptq_master_resident", TORCH_FN(pack_matgptq_master_resident));
+  m.impl("unpack_matgptq_master_resident", TORCH_FN(unpack_matgptq_master_resident));
 }
 
 // On ROCm builds of PyTorch HIP tensors carry the CUDA dispatch key.
 TORCH_LIBRARY_IMPL(matgptq_cuda, CUDA, m) {
   m.impl("matmul_matgptq", TORCH_FN(matmul_matgptq));
   m.impl("matmul_matgptq_zp", TORCH_FN(matmul_matgptq_zp));
+  m.impl("matmul_matgptq_master", TORCH_FN(matmul_matgptq_master));
   m.impl("slice_matgptq_master", TORCH_FN(slice_matgptq_master));
   m.impl("dequantize_matgptq", TORCH_FN(dequantize_matgptq));
 }

@@ -17,6 +17,11 @@ Additive operators of this implementation (all under torch.ops.matgptq_cuda):
     unpack_matgptq_qweights  packed -> uint8 codes (tests, bit-exactness checks)
     slice_matgptq_master     rounded MSB slice of master codes on the GPU
     dequantize_matgptq       packed -> dense fp16 weight, rounded like the reference's dequantize
+    pack_matgptq_master_resident    8-bit master codes [N, K] -> bit planes, most significant first
+                                    (N*K/4 words): one buffer that serves every bitwidth
+    matmul_matgptq_master           matmul_matgptq_zp on those planes with `bitwidth` as a run-time
+                                    argument: the rounded slice is formed in registers
+    unpack_matgptq_master_resident  planes -> the uint8 codes the GEMM sees at `bitwidth`
 """
 from __future__ import annotations
 
@@ -32,6 +37,9 @@ matmul_matgptq_zp = _ops.matmul_matgptq_zp
 unpack_matgptq_qweights = _ops.unpack_matgptq_qweights
 slice_matgptq_master = _ops.slice_matgptq_master
 dequantize_matgptq = _ops.dequantize_matgptq
+pack_matgptq_master_resident = _ops.pack_matgptq_master_resident
+unpack_matgptq_master_resident = _ops.unpack_matgptq_master_resident
+matmul_matgptq_master = _ops.matmul_matgptq_master
 
 
 def _out_dtype(feature_flag: int) -> torch.dtype:
@@ -50,6 +58,13 @@ def _matmul_fake(input, matgptq_weights, matgptq_scales, n_out_features, n_in_fe
 @torch.library.register_fake("matgptq_cuda::matmul_matgptq_zp")
 def _matmul_zp_fake(input, matgptq_weights, matgptq_scales, matgptq_zeros, n_out_features,
                     n_in_features, bitwidth, group_size, feature_flag):
+    m = input.numel() // n_in_features
+    return input.new_empty((m, n_out_features), dtype=_out_dtype(feature_flag))
+
+
+@torch.library.register_fake("matgptq_cuda::matmul_matgptq_master")
+def _matmul_master_fake(input, planes, matgptq_scales, matgptq_zeros, n_out_features, n_in_features,
+                        bitwidth, group_size, feature_flag):
     m = input.numel() // n_in_features
     return input.new_empty((m, n_out_features), dtype=_out_dtype(feature_flag))
 

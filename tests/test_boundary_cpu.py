@@ -29,7 +29,7 @@ def test_python_names_of_the_reference_package():
         assert callable(getattr(matgptq_cuda._CUDA, n))
     import matgptq_cuda._CUDA as ext  # the reference's extension-module name
 
-    assert ext.abi_version() == 1
+    assert ext.abi_version() == 2
     assert (MatGTPQ_FeatureFlags.SYNC, MatGTPQ_FeatureFlags.ASYNC, MatGTPQ_FeatureFlags.IS_BF16) == (0, 1, 2)
     assert set(["matgptq_qweight", "matgptq_scales"]) <= set(MatGPTQLinear.__init__.__code__.co_names) | {"matgptq_qweight", "matgptq_scales"}
 

@@ -27,7 +27,7 @@ def test_every_declared_symbol_is_exported():
     lib = ctypes.CDLL(_lib.ABI_PATH)
     for n in sorted(names):
         assert hasattr(lib, n), n
-    assert L().matgptq_abi_version() == 1
+    assert L().matgptq_abi_version() == 2
 
 
 @pytest.mark.parametrize("b", BITS)

@@ -21,7 +21,12 @@ Differences, all additive:
     reference.  vLLM is not importable in this build's environment: what its loader does with
     these parameters is exercised only through a stand-in loader in the tests;
   * `keep_master_codes` (constructor argument / config key, default false): the 8-bit master
-    codes stay resident after loading and `set_bitwidth` re-slices a layer in place.
+    codes stay resident after loading next to the packed slice and `set_bitwidth` re-slices a
+    layer in place (one device pass over its codes);
+  * `resident_master_planes` (same, default false): ONLY the master codes stay resident, as bit
+    planes (`pack_matgptq_master_resident`), and every product goes through
+    `matmul_matgptq_master`, which slices to the layer's current bitwidth in registers:
+    `set_bitwidth` then changes a number and moves nothing.
 
 vLLM itself is imported lazily: without it the module still imports (the classes then
 derive from small local bases), which is what the CPU test-suite exercises.
@@ -103,6 +108,7 @@ class MatGPTQConfig(QuantizationConfig):
         has_zeros: bool = False,
         has_perm: bool = False,
         keep_master_codes: bool = False,
+        resident_master_planes: bool = False,
     ) -> None:
         super().__init__()
         assert group_size in [-1, 32, 128]
@@ -118,6 +124,9 @@ class MatGPTQConfig(QuantizationConfig):
         self.has_zeros = bool(has_zeros)
         self.has_perm = bool(has_perm)
         self.keep_master_codes = bool(keep_master_codes)
+        self.resident_master_planes = bool(resident_master_planes)
+        if self.resident_master_planes and master_bitwidth != 8:
+            raise ValueError("resident_master_planes needs 8-bit master codes")
         for bits in [inference_bitwidth, *self.layer_bitwidths.values()]:
             if bits not in (2, 3, 4, 6, 8):
                 raise ValueError("bitwidth must be one of {2, 3, 4, 6, 8}")
@@ -150,7 +159,8 @@ class MatGPTQConfig(QuantizationConfig):
         layer_bitwidths = config.get("layer_bitwidths")
         return cls(group_size, master_bitwidth, inference_bitwidth, quant_dtype,
                    modules_to_not_convert, layer_bitwidths, config.get("has_zeros", False),
-                   config.get("has_perm", False), config.get("keep_master_codes", False))
+                   config.get("has_perm", False), config.get("keep_master_codes", False),
+                   config.get("resident_master_planes", False))
 
     def bitwidth_for(self, prefix: str) -> int:
         """Bitwidth of the layer called `prefix`: the longest matching suffix key of
@@ -237,7 +247,13 @@ class MatGPTQLinearMethod(LinearMethodBase):
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         with torch.no_grad():
             qweight = layer.qweight.data
-            layer.matgptq_weights = Parameter(self._pack_at(layer, qweight, self.bitwidth), requires_grad=False)
+            if self.config.resident_master_planes:
+                layer.matgptq_planes = Parameter(
+                    torch.ops.matgptq_cuda.pack_matgptq_master_resident(qweight.contiguous()), requires_grad=False)
+                layer.matgptq_weights = None
+            else:
+                layer.matgptq_planes = None
+                layer.matgptq_weights = Parameter(self._pack_at(layer, qweight, self.bitwidth), requires_grad=False)
             layer.matgptq_bitwidth = self.bitwidth
             layer.matgptq_scales = Parameter(
                 torch.ops.matgptq_cuda.reorder_matgptq_scales(
@@ -258,28 +274,33 @@ class MatGPTQLinearMethod(LinearMethodBase):
             if perm is not None:
                 # act-order: the codes are stored in permuted column order and the input features
                 # are gathered with the permutation (src/quant_utils_matgpqt.py:218-220)
-                layer.matgptq_perm = Parameter(perm.data.to(device=layer.matgptq_weights.device,
+                layer.matgptq_perm = Parameter(perm.data.to(device=layer.matgptq_scales.device,
                                                             dtype=torch.int64).reshape(-1), requires_grad=False)
                 del layer.perm
             else:
                 layer.matgptq_perm = None
 
-            if self.config.keep_master_codes:
+            if self.config.keep_master_codes and not self.config.resident_master_planes:
                 # The reference deletes the master codes here (inference_lib/vllm_matgptq.py:177-178);
                 # kept, a layer can be re-sliced to another bitwidth without the checkpoint.
-                layer.matgptq_master = Parameter(qweight.to(layer.matgptq_weights.device), requires_grad=False)
+                layer.matgptq_master = Parameter(qweight.to(layer.matgptq_scales.device), requires_grad=False)
             del layer.qweight
             del layer.scales
 
     def set_bitwidth(self, layer: torch.nn.Module, bitwidth: int) -> None:
-        """Re-slices a loaded layer to `bitwidth` from its resident master codes (needs
-        `keep_master_codes`).  One device pass over the codes; not for use inside a captured graph
-        (the packed tensor changes size)."""
-        master = getattr(layer, "matgptq_master", None)
-        if master is None:
-            raise RuntimeError("set_bitwidth needs the master codes: load with keep_master_codes")
+        """Moves a loaded layer to `bitwidth`.  With `resident_master_planes` nothing is touched but
+        the number the next product is called with.  With `keep_master_codes` the layer is re-sliced
+        from its resident master codes: one device pass over the codes, not for use inside a captured
+        graph (the packed tensor changes size)."""
         if bitwidth not in (2, 3, 4, 6, 8):
             raise ValueError("bitwidth must be one of {2, 3, 4, 6, 8}")
+        if getattr(layer, "matgptq_planes", None) is not None:
+            layer.matgptq_bitwidth = bitwidth
+            return
+        master = getattr(layer, "matgptq_master", None)
+        if master is None:
+            raise RuntimeError("set_bitwidth needs the master codes: load with keep_master_codes "
+                               "or resident_master_planes")
         with torch.no_grad():
             layer.matgptq_weights = Parameter(self._pack_at(layer, master.data, bitwidth), requires_grad=False)
             layer.matgptq_bitwidth = bitwidth
@@ -289,7 +310,12 @@ class MatGPTQLinearMethod(LinearMethodBase):
         bitwidth = getattr(layer, "matgptq_bitwidth", self.bitwidth)
         if getattr(layer, "matgptq_perm", None) is not None:
             x = torch.index_select(x, -1, layer.matgptq_perm)
-        if getattr(layer, "matgptq_zeros", None) is not None:
+        if getattr(layer, "matgptq_planes", None) is not None:
+            y = torch.ops.matgptq_cuda.matmul_matgptq_master(
+                x, layer.matgptq_planes, layer.matgptq_scales, getattr(layer, "matgptq_zeros", None),
+                self.n_out_features, self.n_in_features, bitwidth,
+                self.config.group_size, self.config.flag)
+        elif getattr(layer, "matgptq_zeros", None) is not None:
             y = torch.ops.matgptq_cuda.matmul_matgptq_zp(
                 x, layer.matgptq_weights, layer.matgptq_scales, layer.matgptq_zeros,
                 self.n_out_features, self.n_in_features, bitwidth,
