@@ -268,6 +268,30 @@ def main() -> int:
                     }
                 del ring
         extra["gemv_M1"] = table
+        # ----------------- master-resident planes: one buffer, bitwidth chosen per call (M = 1)
+        # moved bytes per weight: (b + 1) / 8 for 2, 3 and 4 bits (the top b bits and the round bit),
+        # 1 for 6 and 8 bits; both rates are stated, on the sliced bytes and on the bytes moved
+        mtab = {}
+        for name, (n, k) in LLAMA3_8B.items():
+            words = L.matgptq_master_words(n, k)
+            cp = max(2, int(RING_BYTES // (n * k)) + 1)
+            mring = [torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), dtype=torch.int32, device=dev, generator=g)
+                     for _ in range(cp)]
+            reps = max(cp, 32)
+            for b in (8, 6, 4, 3, 2):
+                def one(i):
+                    _lib.check(L.matgptq_gemm_master(b, GROUP, n, k, 1, mring[i % cp].data_ptr(), aux[name][0].data_ptr(),
+                                                     aux[name][1].data_ptr(), xs[name].data_ptr(), ys[name].data_ptr(),
+                                                     None, 0, stream.cuda_stream, 1))
+                t = timed_graph(lambda: [one(i) for i in range(reps)]) / reps
+                moved = n * k * (b + 1 if b <= 4 else 8) // 8
+                mtab[f"{name}_b{b}"] = {"us": round(t * 1e6, 2),
+                                        "sliced_GBps": round(n * k * b / 8 / t / 1e9, 1),
+                                        "moved_GBps": round(moved / t / 1e9, 1),
+                                        "pct_hbm_peak_moved": round(moved / t / 1e9 / HBM_PEAK_GBPS * 100, 1),
+                                        "presliced_us": table[f"{name}_b{b}_zp"]["us"]}
+            del mring
+        extra["gemv_M1_master_resident"] = mtab
         # ----------------------------------------- small batch (configs[2]), all four layers
         small = {}
         for name, (n, k) in LLAMA3_8B.items():
