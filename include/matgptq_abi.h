@@ -36,6 +36,7 @@ extern "C" {
 #define MATGPTQ_EVARIANT (-7)  /* a forced kernel variant does not apply to this problem */
 #define MATGPTQ_ESIZE (-8)     /* a size exceeds what the entry point supports */
 #define MATGPTQ_EWORKSPACE (-9) /* workspace missing or too small */
+#define MATGPTQ_ESTATIC (-10)   /* needs more than the library's built-in workspace */
 
 /* feature_flag bits: the reference's `Features` word
  * (inference_lib/matgptq_cuda/csrc/include/common.cuh:78-86,
@@ -158,6 +159,21 @@ int matgptq_gemm_master(int bitwidth, int group_size, int64_t N, int64_t K, int6
                         const void *planes_dev, const void *scales_dev, const void *zeros_dev,
                         const void *x_dev, void *y_dev, void *workspace_dev, size_t workspace_bytes,
                         void *stream, uint32_t flags);
+
+/* matgptq_gemm_master without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it is for callers that cannot allocate or carry a workspace along:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Where
+ * matgptq_gemm_master would use its workspace, this entry point uses a buffer of
+ * MATGPTQ_STATIC_WORKSPACE_BYTES that is part of the library's device code (every GPU the library
+ * runs on holds one copy until the process ends).  A shape whose sliced tensor
+ * (bitwidth*N*K/8 bytes) does not fit returns MATGPTQ_ESTATIC.  All calls on one GPU share that
+ * buffer: calls that overlap in time on one GPU (different streams) race, calls on one stream do
+ * not.  The first call on a device looks the buffer's address up (hipGetSymbolAddress), so make
+ * that call outside graph capture. */
+#define MATGPTQ_STATIC_WORKSPACE_BYTES (64u * 1024u * 1024u)
+int matgptq_gemm_master_static(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                               const void *planes_dev, const void *scales_dev, const void *zeros_dev,
+                               const void *x_dev, void *y_dev, void *stream, uint32_t flags);
 
 /* Human-readable name of the kernel variant matgptq_gemm would launch. */
 int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,

@@ -23,7 +23,7 @@ EXPORTS = (
     "matgptq_slice_device", "matgptq_dequantize_device", "matgptq_describe_plan",
     "matgptq_master_words", "matgptq_pack_master_host", "matgptq_pack_master_device",
     "matgptq_unpack_master_host", "matgptq_unpack_master_device",
-    "matgptq_gemm_master_workspace_bytes", "matgptq_gemm_master",
+    "matgptq_gemm_master_workspace_bytes", "matgptq_gemm_master", "matgptq_gemm_master_static",
 )
 
 _lib = None
@@ -83,6 +83,8 @@ def load() -> ctypes.CDLL:
     L.matgptq_gemm_master_workspace_bytes.restype = ctypes.c_size_t
     L.matgptq_gemm_master.argtypes = [ci, ci, i64, i64, i64, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, vp, u32]
     L.matgptq_gemm_master.restype = ci
+    L.matgptq_gemm_master_static.argtypes = [ci, ci, i64, i64, i64, vp, vp, vp, vp, vp, vp, u32]
+    L.matgptq_gemm_master_static.restype = ci
     _lib = L
     return L
 

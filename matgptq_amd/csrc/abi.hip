@@ -6,9 +6,15 @@
 
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/matgptq_abi.h"
 #include "device_common.h"
+
+// Scratch of matgptq_gemm_master_static: device memory that lives in the library's code object, so
+// that entry point needs no allocation at all.  One copy per GPU, at its own address.
+constexpr size_t kStaticScratchBytes = (size_t)MATGPTQ_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace matgptq {
 
@@ -357,6 +363,9 @@ const char* matgptq_strerror(int code) {
     case MATGPTQ_EVARIANT: return "forced kernel variant does not apply to this problem";
     case MATGPTQ_ESIZE: return "size exceeds the supported maximum";
     case MATGPTQ_EWORKSPACE: return "workspace missing or smaller than matgptq_gemm_master_workspace_bytes()";
+    case MATGPTQ_ESTATIC:
+      return "the sliced tensor is larger than the library's built-in workspace (MATGPTQ_STATIC_WORKSPACE_BYTES): "
+             "use matgptq_gemm_master with a workspace";
     default: return "unknown error";
   }
 }
@@ -451,6 +460,40 @@ int matgptq_gemm_master(int bitwidth, int group_size, int64_t N, int64_t K, int6
                         void* stream, uint32_t flags) {
   return gemm_master_impl(bitwidth, group_size, N, K, M, planes_dev, scales_dev, zeros_dev, x_dev, y_dev,
                           workspace_dev, workspace_bytes, stream, flags);
+}
+
+// Address of this GPU's copy of `scratch`: looked up once per device, with that device current
+// (the array's name is only a host-side handle, not a device address).
+static int static_scratch(void** ptr) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static void* addr[kMaxDevices] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MATGPTQ_ELAUNCH;
+  std::lock_guard<std::mutex> guard(lock);
+  if (addr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return MATGPTQ_ELAUNCH;
+    addr[dev] = p;
+  }
+  *ptr = addr[dev];
+  return MATGPTQ_OK;
+}
+
+int matgptq_gemm_master_static(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                               const void* planes_dev, const void* scales_dev, const void* zeros_dev,
+                               const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
+  bool direct = false;
+  if (int e = master_reads_planes(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &direct)) return e;
+  void* ws = nullptr;
+  size_t need = 0;
+  if (!direct) {
+    need = matgptq_packed_words(bitwidth, N, K) * 4;
+    if (need > kStaticScratchBytes) return MATGPTQ_ESTATIC;
+    if (int e = static_scratch(&ws)) return e;
+  }
+  return gemm_master_impl(bitwidth, group_size, N, K, M, planes_dev, scales_dev, zeros_dev, x_dev, y_dev, ws,
+                          need, stream, flags);
 }
 
 int matgptq_pack_master_device(const uint8_t* codes_dev, int64_t N, int64_t K, uint32_t* planes_dev,
