@@ -134,15 +134,14 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       const int nb = prefill_tail_big_tiles(row_blocks, m_tiles);
       const int64_t rest = (int64_t)((row_blocks - nb * 16 + 15) / 16) * m_tiles;
       if (nb > 0 && rest > 0 && rest <= 256) p->cfg = 8;
-      // Two register sets of 6-bit codes (and of 8-bit codes with zero points) for four row
-      // blocks do not fit beside the accumulators of the 128 x 256 tile: it spills and runs at
-      // half the rate of the 128 x 128 ring tile (8192 x 8192, M = 2048, 6 bits: 596 against
-      // 281 us; 8 bits with zero points: 316 against 269 us).
+      // 6-bit codes for four row blocks do not fit beside the accumulators of the 128 x 256 tile even
+      // with a single set refilled octet by octet (as 8-bit codes are): it spills and runs at half the
+      // rate of the 128 x 128 ring tile (8192 x 8192, M = 2048, 6 bits: 596 against 281 us).
       // Between the two, a 128 x 192 tile (three row blocks per wave) fits the registers and runs
       // about 9 % faster per weight than the 128 x 128 tile where its tiles fill the rounds of 512
       // resident workgroups as well (57344 x 8192, 6 bits: 1748 against 1906 us; on 8192 rows, 43
       // tiles of 192, it only ties).  Rounds times tile width decide.
-      if (bits == 6 || (bits == 8 && zp)) {
+      if (bits == 6) {
         const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
         const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
         const double t_128 = (double)((wgs_128 + 511) / 512);

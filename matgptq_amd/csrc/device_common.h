@@ -128,13 +128,14 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t o
 template <int BITS>
 struct UnpackConsts {
   uint32_t magic;  // VGPR: two fp16 1024.0
-  uint32_t m[3];   // SGPRs: field masks
+  uint32_t m[4];   // SGPRs: field masks
   __device__ __forceinline__ UnpackConsts() {
     magic = opaque_vgpr(kMagic);
     if constexpr (BITS == 2) {
       m[0] = opaque_sgpr(0x00030003u); m[1] = opaque_sgpr(0x000C000Cu); m[2] = opaque_sgpr(0x00300030u);
     } else if constexpr (BITS == 6) {
-      m[0] = opaque_sgpr(0x00030003u); m[1] = opaque_sgpr(0x00300030u); m[2] = 0;
+      m[0] = opaque_sgpr(0x00030003u); m[1] = opaque_sgpr(0x00300030u);
+      m[2] = opaque_sgpr(0x003C003Cu); m[3] = opaque_sgpr(0x03C003C0u);
     } else if constexpr (BITS == 3) {
       m[0] = opaque_sgpr(0x000F000Fu); m[1] = opaque_sgpr(0x00F000F0u); m[2] = opaque_sgpr(0x44444444u);
     } else {
@@ -179,13 +180,18 @@ __device__ __forceinline__ void raw_octet(const uint32_t (&w)[BITS], const Unpac
       r[3] = and_or(x12, k.m[1], k.magic);
     }
   } else if constexpr (BITS == 6) {
-    const uint32_t h = w[J], h8 = h >> 8;
+    // high nibbles shifted to bits 2..5 of their fields once per word (<< 2 for pairs 0, 1; >> 6 for
+    // pairs 2, 3, whose nibbles sit 8 bits higher); a pair is then two v_and_or_b32: the low bits
+    // over the magic word, the high nibble over that (their bit ranges are disjoint)
+    const uint32_t hs = w[J] << 2, hs6 = w[J] >> 6;
     const uint32_t l = (J & 1) ? (w[4 + (J >> 1)] >> 8) : w[4 + (J >> 1)];
     const uint32_t l2 = l >> 2;
-    r[0] = ((h & 0x000F000Fu) << 2) | and_or(l, k.m[0], k.magic);
-    r[1] = ((h & 0x00F000F0u) << 2) | and_or(l, k.m[1], k.magic);
-    r[2] = ((h8 & 0x000F000Fu) << 2) | and_or(l2, k.m[0], k.magic);
-    r[3] = ((h8 & 0x00F000F0u) << 2) | and_or(l2, k.m[1], k.magic);
+    // (the inner result is hidden from the optimiser, which would otherwise regroup the two
+    // v_and_or_b32 of a pair into two v_and_b32 and a v_or3_b32)
+    r[0] = and_or(hs, k.m[2], opaque_vgpr(and_or(l, k.m[0], k.magic)));
+    r[1] = and_or(hs, k.m[3], opaque_vgpr(and_or(l, k.m[1], k.magic)));
+    r[2] = and_or(hs6, k.m[2], opaque_vgpr(and_or(l2, k.m[0], k.magic)));
+    r[3] = and_or(hs6, k.m[3], opaque_vgpr(and_or(l2, k.m[1], k.magic)));
   } else {
     // bytes: pair 2d = (byte0, byte2) of word 2J+d, pair 2d+1 = (byte1, byte3)
     const uint32_t fill = 0x64646464u;

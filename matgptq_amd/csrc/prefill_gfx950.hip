@@ -63,6 +63,33 @@ constexpr int prefill_lds_halves(int rbw, int mt) {
   return prefill_lean(rbw, mt) ? 4 * 16 * mt * kXs : 2 * 16 * mt * kXsPitch;
 }
 
+// Wide codes on the 128 x 256 tile: two register sets of 6-bit codes (or of 8-bit codes next to
+// zero points) for four row blocks do not fit beside the 128 accumulators.  Those formats keep ONE
+// set and refill the words of an octet with the next tile's right after the octet has been
+// dequantised (three 32-column steps before they are needed again), one small load per octet.
+constexpr bool prefill_streams_codes(int bits, bool zp, int rbw, int mt) {
+  (void)zp;
+  return !kBf16 && rbw == 4 && mt == 8 && (bits == 6 || bits == 8);
+}
+// loads refill_octet issues for octet j
+constexpr int refill_loads(int bits, int j) { return bits == 6 && (j & 1) ? 2 : 1; }
+
+// The words octet J of a lane is decoded from, out of the tile at `tile_off` (8 bits: words 2J, 2J+1;
+// 6 bits: word J and, behind the odd octets, the word of low bits they share with their neighbour).
+template <int BITS, int J>
+__device__ __forceinline__ void refill_octet(BufRsrc rs, uint32_t tile_off, int lane, uint32_t (&w)[BITS]) {
+  static_assert(BITS == 6 || BITS == 8, "wide codes only");
+  if constexpr (BITS == 8) {
+    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rs, (J >> 1) * 1024 + lane * 16 + (J & 1) * 8, tile_off, 0);
+    w[2 * J] = v.x;
+    w[2 * J + 1] = v.y;
+  } else {
+    w[J] = __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 16 + J * 4, tile_off, 0);
+    if constexpr ((J & 1) != 0)
+      w[4 + (J >> 1)] = __builtin_amdgcn_raw_buffer_load_b32(rs, 1024 + lane * 8 + (J >> 1) * 4, tile_off, 0);
+  }
+}
+
 // One workgroup tile: activation rows [mtile * 16 MT, +16 MT) x the weight rows of the row blocks
 // rb_base + [nt * 4 RBW, +4 RBW), where lid = nt * m_tiles + mtile.  `lds` is the workgroup's
 // LDS (prefill_lds_halves(RBW, MT) halves, 16-byte aligned).
@@ -302,38 +329,120 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     using J1 = std::integral_constant<int, 1>;
     using J2 = std::integral_constant<int, 2>;
     using J3 = std::integral_constant<int, 3>;
-    // buffer loads one load_weights() issues: the codes, then a scale (and a zero) per group
-    constexpr int kW = RBW * tile_load_count(BITS) + RBW * GPT * (ZP ? 2 : 1);
-    // issue order of the wave's buffer loads: prologue  D0 D1 D2 D3 W0 W1 ; then per tile t
-    //   after the first barrier D(2t+4), after the second barrier D(2t+5), at its end W(t+2)
-    // (D = 4 copies of one half tile, W = kW loads of one tile's codes, scales and zeros)
-    dma(ring0, 0);
-    dma(ring1, 1);
-    dma(ring2, 2);
-    dma(ring3, 3);
-    load_weights(wcur, scur, zcur, 0);
-    load_weights(wnxt, snxt, znxt, 1);
-    wait_and_meet(std::integral_constant<int, 12 + 2 * kW>{});  // D0 has landed
+    if constexpr (prefill_streams_codes(BITS, ZP, RBW, MT)) {
+      // ---- one set of codes, refilled octet by octet; scales and zeros keep their two sets ----
+      // loads per refill of octet J for all row blocks, and per set of scales (and zeros)
+      constexpr int r0 = RBW * refill_loads(BITS, 0), r1 = RBW * refill_loads(BITS, 1);
+      constexpr int r2 = RBW * refill_loads(BITS, 2), r3 = RBW * refill_loads(BITS, 3);
+      constexpr int kS = RBW * GPT * (ZP ? 2 : 1);
+      auto refill = [&](auto jtag, int kb) {  // octet J of tile kb into the one set of codes
+        constexpr int J = decltype(jtag)::value;
 #pragma unroll
-    for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
-    // one tile; ra / rb: the rings of its two half tiles, rn: the ring of the next tile's first
-    auto dtile = [&](int kb, uint32_t (&wc)[RBW][BITS], uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT],
-                     _Float16* ra, _Float16* rb, _Float16* rn) {
-      dstep(wc, sc, zc, J0{}, ra, 1);
-      // needs D(2kb+1); younger in steady state: W(kb) D(2kb+2) D(2kb+3) W(kb+1)
-      wait_and_meet(std::integral_constant<int, 8 + 2 * kW>{});
-      dma(ra, 2 * kb + 4);  // every wave is past its reads of ra
-      dstep(wc, sc, zc, J1{}, rb, 0);
-      dstep(wc, sc, zc, J2{}, rb, 1);
-      // needs D(2kb+2); younger: D(2kb+3) W(kb+1) D(2kb+4)
-      wait_and_meet(std::integral_constant<int, 8 + kW>{});
-      dma(rb, 2 * kb + 5);
-      dstep(wc, sc, zc, J3{}, rn, 0);
-      load_weights(wc, sc, zc, kb + 2);  // this set is free now
-    };
-    for (int kb = 0; kb < a.k_tiles; kb += 2) {
-      dtile(kb, wcur, scur, zcur, ring0, ring1, ring2);
-      if (kb + 1 < a.k_tiles) dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
+        for (int rr = 0; rr < RBW; rr++) {
+          const int rb = rb_first + rr;
+          const bool valid = rb < a.row_blocks && kb < a.k_tiles;
+          const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
+          refill_octet<BITS, J>(wr, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, wcur[rr]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      auto load_aux = [&](uint32_t (&sv)[RBW][GPT], uint32_t (&zv)[RBW][GPT], int kb) {
+#pragma unroll
+        for (int rr = 0; rr < RBW; rr++) {
+          const int rb = rb_first + rr;
+          const bool valid = rb < a.row_blocks && kb < a.k_tiles;
+          const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
+          const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
+#pragma unroll
+          for (int gg = 0; gg < GPT; gg++) {
+            const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
+            const uint32_t so = ((uint32_t)rb * a.G + g) * 32;
+            sv[rr][gg] = __builtin_amdgcn_raw_buffer_load_b16(sr, r16 * 2, so, 0);
+            if constexpr (ZP) zv[rr][gg] = __builtin_amdgcn_raw_buffer_load_b16(zr, r16 * 2, so, 0);
+            else zv[rr][gg] = 0u;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // Issue order of the wave's buffer loads (D = 4 copies of a half tile, Rj = refill of octet j,
+      // S = scales and zeros of a tile):
+      //   prologue  D0 D1 D2 D3  R0(0) R1(0) R2(0) R3(0)  S(0) S(1)
+      //   tile t    [octet 0] R0(t+1) | barrier A, D(2t+4) | [1] R1(t+1) [2] R2(t+1) | barrier B, D(2t+5) |
+      //             [3] R3(t+1) S(t+2)
+      // Barrier A of tile t needs D(2t+1), issued behind barrier B of tile t-2; issued after it:
+      //   R3 S | R0 D R1 R2 D R3 S | R0, and at t = 0 (D1 from the prologue): D2 D3 R0..R3 S S | R0, which is
+      //   r3 loads fewer: the smaller count is used for every tile (a stricter wait, on loads that are
+      //   more than a tile old).  Barrier B of tile t needs D(2t+2), issued behind barrier A of tile t-1;
+      //   issued after it: R1 R2 D R3 S | R0 D R1 R2 (more at t = 0).
+      constexpr int kWaitA = 8 + 2 * r0 + r1 + r2 + r3 + 2 * kS;
+      constexpr int kWaitB = 8 + r0 + 2 * r1 + 2 * r2 + r3 + kS;
+      dma(ring0, 0);
+      dma(ring1, 1);
+      dma(ring2, 2);
+      dma(ring3, 3);
+      refill(J0{}, 0);
+      refill(J1{}, 0);
+      refill(J2{}, 0);
+      refill(J3{}, 0);
+      load_aux(scur, zcur, 0);
+      load_aux(snxt, znxt, 1);
+      wait_and_meet(std::integral_constant<int, 12 + r0 + r1 + r2 + r3 + 2 * kS>{});  // D0 has landed
+#pragma unroll
+      for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
+      auto stile = [&](int kb, uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT], _Float16* ra, _Float16* rb,
+                       _Float16* rn) {
+        dstep(wcur, sc, zc, J0{}, ra, 1);
+        refill(J0{}, kb + 1);
+        wait_and_meet(std::integral_constant<int, kWaitA>{});
+        dma(ra, 2 * kb + 4);
+        dstep(wcur, sc, zc, J1{}, rb, 0);
+        refill(J1{}, kb + 1);
+        dstep(wcur, sc, zc, J2{}, rb, 1);
+        refill(J2{}, kb + 1);
+        wait_and_meet(std::integral_constant<int, kWaitB>{});
+        dma(rb, 2 * kb + 5);
+        dstep(wcur, sc, zc, J3{}, rn, 0);
+        refill(J3{}, kb + 1);
+        load_aux(sc, zc, kb + 2);  // this set is free now
+      };
+      for (int kb = 0; kb < a.k_tiles; kb += 2) {
+        stile(kb, scur, zcur, ring0, ring1, ring2);
+        if (kb + 1 < a.k_tiles) stile(kb + 1, snxt, znxt, ring2, ring3, ring0);
+      }
+    } else {
+    // buffer loads one load_weights() issues: the codes, then a scale (and a zero) per group
+      constexpr int kW = RBW * tile_load_count(BITS) + RBW * GPT * (ZP ? 2 : 1);
+      // issue order of the wave's buffer loads: prologue  D0 D1 D2 D3 W0 W1 ; then per tile t
+      //   after the first barrier D(2t+4), after the second barrier D(2t+5), at its end W(t+2)
+      // (D = 4 copies of one half tile, W = kW loads of one tile's codes, scales and zeros)
+      dma(ring0, 0);
+      dma(ring1, 1);
+      dma(ring2, 2);
+      dma(ring3, 3);
+      load_weights(wcur, scur, zcur, 0);
+      load_weights(wnxt, snxt, znxt, 1);
+      wait_and_meet(std::integral_constant<int, 12 + 2 * kW>{});  // D0 has landed
+  #pragma unroll
+      for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
+      // one tile; ra / rb: the rings of its two half tiles, rn: the ring of the next tile's first
+      auto dtile = [&](int kb, uint32_t (&wc)[RBW][BITS], uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT],
+                       _Float16* ra, _Float16* rb, _Float16* rn) {
+        dstep(wc, sc, zc, J0{}, ra, 1);
+        // needs D(2kb+1); younger in steady state: W(kb) D(2kb+2) D(2kb+3) W(kb+1)
+        wait_and_meet(std::integral_constant<int, 8 + 2 * kW>{});
+        dma(ra, 2 * kb + 4);  // every wave is past its reads of ra
+        dstep(wc, sc, zc, J1{}, rb, 0);
+        dstep(wc, sc, zc, J2{}, rb, 1);
+        // needs D(2kb+2); younger: D(2kb+3) W(kb+1) D(2kb+4)
+        wait_and_meet(std::integral_constant<int, 8 + kW>{});
+        dma(rb, 2 * kb + 5);
+        dstep(wc, sc, zc, J3{}, rn, 0);
+        load_weights(wc, sc, zc, kb + 2);  // this set is free now
+      };
+      for (int kb = 0; kb < a.k_tiles; kb += 2) {
+        dtile(kb, wcur, scur, zcur, ring0, ring1, ring2);
+        if (kb + 1 < a.k_tiles) dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
+      }
     }
   } else {
   Frag awA[RBW], awB[RBW];

@@ -167,15 +167,16 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
         _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8))
 
 
-def test_planner_keeps_wide_codes_off_the_largest_ring_tile():
-    # two register sets of 6-bit codes (8-bit with zero points) spill in the 128 x 256 tile
+def test_planner_keeps_six_bit_codes_off_the_largest_ring_tile():
+    # 6-bit codes spill in the 128 x 256 tile; 8-bit codes keep one set there, refilled octet by octet
     assert _lib.describe_plan(6, 128, 8192, 8192, 2048, True).endswith("cfg3")
     assert _lib.describe_plan(6, 128, 28672 // 4, 8192, 2048, False).endswith("cfg3")
     assert _lib.describe_plan(6, 128, 10240, 8192, 2048, False).endswith("cfg9")  # 54 tiles of 192 rows: two rounds
     # many rounds: the 128 x 192 tile, which still fits the registers
     assert _lib.describe_plan(6, 128, 57344, 8192, 2048, True).endswith("cfg9")
-    assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True).endswith("cfg9")
+    assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(8, 128, 57344, 8192, 2048, False).endswith("cfg0")
-    assert _lib.describe_plan(8, 128, 8192, 8192, 2048, True).endswith("cfg3")
+    assert _lib.describe_plan(8, 128, 8192, 8192, 2048, True).endswith("cfg0")
+    assert _lib.describe_plan(8, 128, 10240, 8192, 2048, True).endswith("cfg8")
     assert _lib.describe_plan(8, 128, 8192, 8192, 2048, False).endswith("cfg0")
     assert _lib.describe_plan(3, 128, 8192, 8192, 2048, True).endswith("cfg0")
