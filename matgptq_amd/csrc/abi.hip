@@ -123,9 +123,9 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   if (!p->decode) {
     // M > 16.  The 128 x 256 tile (two waves per SIMD, activations copied straight into LDS)
     // once its workgroups fill more than half of the 512 resident slots (measured on MI355X,
-    // Llama-3-8B and 70B layers; bf16 storage has no ring loop, its 128 x 256 tile runs one wave per SIMD).
+    // Llama-3-8B and 70B layers).
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
-    if (wgs_big >= 288 && !(flags & MATGPTQ_FLAG_BF16)) {
+    if (wgs_big >= 288) {
       p->cfg = 0;
       // Whole rounds of 512 resident workgroups plus at most half a round: the rows of that
       // fraction go to 128 x 128 tiles, which run last, one per CU, in about a third of a
@@ -141,11 +141,16 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // about 9 % faster per weight than the 128 x 128 tile where its tiles fill the rounds of 512
       // resident workgroups as well (57344 x 8192, 6 bits: 1748 against 1906 us; on 8192 rows, 43
       // tiles of 192, it only ties).  Rounds times tile width decide.
-      if (bits == 6) {
+      // bf16 storage dequantises through fp32 for the bf16 matrix instruction (four vector
+      // instructions per pair of weights instead of two): the wider tiles spill or stall on that
+      // work, the 128 x 128 tile does not, and up to 4 bits neither does the 128 x 192 tile
+      // (Llama-3-70B gate_up, M = 2048, 4 bits: 1590 against 1768 us; the 128 x 256 tile takes 2241).
+      const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
+      if (bits == 6 || bf16) {
         const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
         const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
         const double t_128 = (double)((wgs_128 + 511) / 512);
-        p->cfg = t_192 < t_128 ? 9 : 3;
+        p->cfg = t_192 < t_128 && (bits <= 4 || !bf16) ? 9 : 3;
       }
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
@@ -234,7 +239,6 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
       if (variant - 64 > 9) return MATGPTQ_EVARIANT;
-      if (variant - 64 == 8 && (flags & MATGPTQ_FLAG_BF16)) return MATGPTQ_EVARIANT;  // ring loop: fp16 storage only
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 64;

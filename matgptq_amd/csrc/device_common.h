@@ -42,9 +42,10 @@ __device__ __forceinline__ half2v h2_from_bits(uint32_t u) {
 }
 
 // ---- bfloat16 storage (activations, scales, zeros, output when the BF16 flag is set) ----
-// The kernels compute in fp16 operands / fp32 accumulators either way; bf16 values are
-// converted where they enter and leave.  bf16 -> fp16 is exact inside fp16's normal range
-// (8 significant bits into 11); magnitudes above 65504 saturate to +-65504.
+// The decode-regime kernels compute in fp16 operands / fp32 accumulators either way; bf16 values
+// are converted where they enter and leave.  bf16 -> fp16 is exact inside fp16's normal range
+// (8 significant bits into 11); magnitudes above 65504 saturate to +-65504.  The prefill kernel
+// multiplies bf16 by bf16 on the matrix cores (no conversion of the activations, no saturation).
 #ifndef MATGPTQ_BF16
 #define MATGPTQ_BF16 0
 #endif
@@ -250,6 +251,36 @@ __device__ __forceinline__ void dequant_octet(const uint32_t (&w)[BITS], const U
   a.p[1] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 1), ZP>(raw[1], zrel, scale);
   a.p[2] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 2), ZP>(raw[2], zrel, scale);
   a.p[3] = dequant_pair<BITS, Codec<BITS>::raw_shift(J, 3), ZP>(raw[3], zrel, scale);
+}
+
+// bf16 storage on the matrix cores' bf16 path (the prefill kernel): the weight is formed in fp32,
+//   w = bf16(fma(u, scale m, -(scale zrel))),  `sm` = scale m, `sz` = scale zrel,
+// one fused conversion and multiply-add per element and one packed conversion per pair.  u (8 bits),
+// a bf16 scale (8 bits) and an integer zero point (8 bits) make both products and their difference
+// exact in fp32, so w is scale (m c - zero) rounded once: the value dequantize() gives on bfloat16
+// tensors whenever m c - zero is itself a bfloat16 (always, for integer zero points).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+
+template <int BITS, int P>
+__device__ __forceinline__ uint32_t dequant_pair_bf16(uint32_t raw, float sm, float sz) {
+  const half2v u = centre_raw<P>(raw, Codec<BITS>::kCentre);
+  // (symmetric layers pass an opaque zero as `sz`: the fused form is one instruction per element,
+  // a conversion followed by a multiplication two)
+  const float2v w = {__builtin_fmaf((float)u.x, sm, -sz), __builtin_fmaf((float)u.y, sm, -sz)};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));
+}
+
+template <int BITS, int J>
+__device__ __forceinline__ void dequant_octet_bf16(const uint32_t (&w)[BITS], const UnpackConsts<BITS>& k,
+                                                   float sm, float sz, Frag& a) {
+  uint32_t raw[4];
+  raw_octet<BITS, J>(w, k, raw);
+  a.u[0] = dequant_pair_bf16<BITS, Codec<BITS>::raw_shift(J, 0)>(raw[0], sm, sz);
+  a.u[1] = dequant_pair_bf16<BITS, Codec<BITS>::raw_shift(J, 1)>(raw[1], sm, sz);
+  a.u[2] = dequant_pair_bf16<BITS, Codec<BITS>::raw_shift(J, 2)>(raw[2], sm, sz);
+  a.u[3] = dequant_pair_bf16<BITS, Codec<BITS>::raw_shift(J, 3)>(raw[3], sm, sz);
 }
 
 // Buffer resources: a 128-bit scalar descriptor (base, byte size) lets every load

@@ -22,6 +22,8 @@
 //    that read it have been issued, every global load is branch-free (tiles beyond K or N go
 //    through a zero-length buffer descriptor), and scales and zeros stay in registers as
 //    loaded (converted at use), so that nothing waits on a load right after issuing it;
+//  * bf16 storage runs the same loops on the bf16 matrix instruction: the activations stay as
+//    stored, the weights are formed in fp32 and rounded to bf16 once (see dequant_pair_bf16);
 //  * fp32 accumulators live in registers for the whole K loop; the epilogue packs
 //    four consecutive output columns per lane into one 8-byte store.
 //
@@ -52,9 +54,7 @@ constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 // Two waves per SIMD (256 registers each) whenever the accumulators leave room for the rest:
 // one wave alone cannot keep the matrix pipe busy.  The tile whose accumulators take half of
 // that budget runs the ring loop below (activations straight into LDS, one operand set).
-// (bf16 storage: the copy into LDS would bypass the bf16 -> fp16 conversion, so that build keeps
-// the staged loop for this tile as well)
-constexpr bool prefill_lean(int rbw, int mt) { return !kBf16 && (rbw == 4 || rbw == 3 || rbw == 2) && mt == 8; }
+constexpr bool prefill_lean(int rbw, int mt) { return (rbw == 4 || rbw == 3 || rbw == 2) && mt == 8; }
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
 // LDS of a workgroup, in halves: the ring loop keeps four unpadded buffers of 64 columns, the
@@ -69,7 +69,7 @@ constexpr int prefill_lds_halves(int rbw, int mt) {
 // dequantised (three 32-column steps before they are needed again), one small load per octet.
 constexpr bool prefill_streams_codes(int bits, bool zp, int rbw, int mt) {
   (void)zp;
-  return !kBf16 && rbw == 4 && mt == 8 && (bits == 6 || bits == 8);
+  return rbw == 4 && mt == 8 && (bits == 6 || bits == 8);
 }
 // loads refill_octet issues for octet j
 constexpr int refill_loads(int bits, int j) { return bits == 6 && (j & 1) ? 2 : 1; }
@@ -126,6 +126,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     for (int mt = 0; mt < MT; mt++) acc[rr][mt] = float4v{0.f, 0.f, 0.f, 0.f};
 
   const UnpackConsts<BITS> kc_unpack;
+  const float kc_zero = __uint_as_float(opaque_vgpr(0u));  // a zero the optimiser cannot see through
   uint32_t wcur[RBW][BITS], wnxt[RBW][BITS];
   // scales and zeros as loaded (16 bits in a register each): converted where they are used, so
   // that nothing has to wait for these loads right after they are issued
@@ -179,7 +180,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
   auto store_x = [&](const u32x4 (&xr)[XCHUNKS], int buf) {
 #pragma unroll
     for (int c = 0; c < XCHUNKS; c++)
-      *reinterpret_cast<half8*>(&xs[buf * kXsBuf + x_lds[c]]) = storage8_to_half8(__builtin_bit_cast(half8, xr[c]));
+      *reinterpret_cast<u32x4*>(&xs[buf * kXsBuf + x_lds[c]]) = xr[c];  // as stored: fp16 or bf16
   };
 
   auto dequant_step = [&](Frag (&aw)[RBW], const uint32_t (&w)[RBW][BITS], const uint32_t (&s)[RBW][GPT],
@@ -188,21 +189,32 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
       const int gg = GROUP == 32 ? J : 0;
-      // fp16 storage: scale * 2^(8-b) and scale * (zero - 128);
-      // bf16 storage: scale * 2^8 and (zero - 128) * 2^-8, converted through fp32
-      _Float16 s1, z1 = (_Float16)0.f;
       if constexpr (kBf16) {
-        s1 = (_Float16)(bf16_bits_to_float(s[rr][gg]) * 256.0f);
-        if constexpr (ZP) z1 = (_Float16)((bf16_bits_to_float(z[rr][gg]) - 128.0f) * (1.0f / 256.0f));
+        // bf16 storage: scale * 2^(8-b) and scale * (zero - 128) in fp32, weights for the bf16 MFMA
+        const float s0 = bf16_bits_to_float(s[rr][gg]);
+        const float sm = s0 * (float)(1 << (8 - BITS));
+        float sz = kc_zero;
+        if constexpr (ZP) sz = s0 * (bf16_bits_to_float(z[rr][gg]) - 128.0f);
+        dequant_octet_bf16<BITS, J>(w[rr], kc_unpack, sm, sz, aw[rr]);
       } else {
+        // fp16 storage: scale * 2^(8-b) and scale * (zero - 128)
         const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)s[rr][gg]);
-        s1 = (_Float16)((float)s0 * (float)(1 << (8 - BITS)));  // scale * m
+        const _Float16 s1 = (_Float16)((float)s0 * (float)(1 << (8 - BITS)));  // scale * m
+        _Float16 z1 = (_Float16)0.f;
         if constexpr (ZP) z1 = s0 * (__builtin_bit_cast(_Float16, (uint16_t)z[rr][gg]) - (_Float16)128.0f);
+        const half2v sc = {s1, s1};
+        const half2v zr = {z1, z1};
+        dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
       }
-      const half2v sc = {s1, s1};
-      const half2v zr = {z1, z1};
-      dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
     }
+  };
+  // one MFMA 16x16x32 in the storage type: weights and activations are both fp16, or both bf16
+  auto mma = [](const Frag& wa, const Frag& xb, float4v c) {
+    if constexpr (kBf16)
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wa.h), __builtin_bit_cast(bf16x8, xb.h),
+                                                     c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(wa.h, xb.h, c, 0, 0, 0);
   };
   auto read_frag = [&](Frag& b, int i, int buf, int jj) {
     b.v = *reinterpret_cast<const uint4*>(&xs[buf * kXsBuf + (i * 16 + r16) * kXsPitch + jj * 32 + q * 8]);
@@ -218,7 +230,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     for (int i = 0; i < MT; i++) {
 #pragma unroll
       for (int rr = 0; rr < RBW; rr++)
-        acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b[i].h, acc[rr][i], 0, 0, 0);
+        acc[rr][i] = mma(aw[rr], b[i], acc[rr][i]);
       read_frag(b[i], i, nbuf, njj);
     }
     constexpr int kValuPerMfma = (RBW * 24 + RBW * MT - 1) / (RBW * MT);
@@ -299,13 +311,13 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       for (int i = 0; i < MT; i++) {
 #pragma unroll
         for (int rr = 0; rr < RBW / 2; rr++)
-          acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, bv[i].h, acc[rr][i], 0, 0, 0);
+          acc[rr][i] = mma(aw[rr], bv[i], acc[rr][i]);
       }
 #pragma unroll
       for (int i = 0; i < MT; i++) {
 #pragma unroll
         for (int rr = RBW / 2; rr < RBW; rr++)
-          acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, bv[i].h, acc[rr][i], 0, 0, 0);
+          acc[rr][i] = mma(aw[rr], bv[i], acc[rr][i]);
         ring_frag(bv[i], nring, i, njj);
       }
       constexpr int kHalf = (RBW / 2) * MT;              // MFMAs of the first half
@@ -626,18 +638,14 @@ prefill_tail_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
 
 template <int GROUP, bool ZP>
 hipError_t launch_tail(const GemmArgs& a, hipStream_t stream) {
-  if constexpr (kBf16) {
-    return hipErrorInvalidValue;  // (bf16 storage has no ring loop)
-  } else {
-    const int m_tiles = (a.M + 127) / 128;
-    const int nb = prefill_tail_big_tiles(a.row_blocks, m_tiles);
-    const int rb_tail = nb * 16;
-    const int n_small = (a.row_blocks - rb_tail + 7) / 8;
-    const dim3 grid((nb + n_small) * m_tiles), block(256);
-    hipLaunchKernelGGL((prefill_tail_kernel<kBits, GROUP, ZP>), grid, block, 0, stream, a, m_tiles,
-                       nb * m_tiles, rb_tail);
-    return hipGetLastError();
-  }
+  const int m_tiles = (a.M + 127) / 128;
+  const int nb = prefill_tail_big_tiles(a.row_blocks, m_tiles);
+  const int rb_tail = nb * 16;
+  const int n_small = (a.row_blocks - rb_tail + 7) / 8;
+  const dim3 grid((nb + n_small) * m_tiles), block(256);
+  hipLaunchKernelGGL((prefill_tail_kernel<kBits, GROUP, ZP>), grid, block, 0, stream, a, m_tiles,
+                     nb * m_tiles, rb_tail);
+  return hipGetLastError();
 }
 
 template <int GROUP, bool ZP, int RBW, int MT>

@@ -322,8 +322,9 @@ def _gemm_bf16(b, g, n, k, x_f32, packed, s_f32, z_f32, flags=3):
 
 
 # One bfloat16 rounding of the output is 2^-9 relative; the oracle additionally rounds every
-# weight to bfloat16 (2^-9 each, independent), which the kernels do not (they keep fp16 weights /
-# exact products).  Bar: max error <= 1e-2 of the largest output, as for fp16.
+# weight to bfloat16 (2^-9 each, independent), which the decode-regime kernels do not (they keep
+# fp16 weights / exact products; the prefill kernel does round them, see the identity test below).
+# Bar: max error <= 1e-2 of the largest output, as for fp16.
 @pytest.mark.parametrize("b", BITS)
 def test_bf16_forward_against_reference_vectors(b, golden):
     n, k = golden["q"].shape
@@ -408,9 +409,28 @@ def test_bf16_midbatch_kernel(b, g, zp):
         assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref)), (b, g, zp, rsel)
 
 
-@pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8)))
+@pytest.mark.parametrize("b", (2, 3, 4, 6, 8))
+@pytest.mark.parametrize("zp", (True, False))
+def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
+    # The prefill kernel multiplies bf16 by bf16 on the matrix cores.  With the identity as
+    # activations every output is one weight (plus exact zeros), so the result must be
+    # dequantize() on bfloat16 tensors, bit for bit (integer zero points: one rounding on both
+    # sides).  Ring tiles 128 x 256, 128 x 128, 128 x 192, the tail split and a staged tile.
+    n, k, g = 304, 256, 128
+    q, s16, z16 = o.make_layer(n, k, g, seed=300 + b, symmetric=not zp)
+    s = o.round_to_bf16(s16.astype(np.float32))
+    z = np.round(z16.astype(np.float32))
+    x = np.eye(k, dtype=np.float32)
+    pk = G.pack_device(q, b, True)
+    w = o.dequantize_bf16(q, s, z, b, g)
+    for cfg in (64, 67, 73, 72, 66):
+        y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | (cfg << 8))
+        assert np.array_equal(y, w.T), (b, zp, cfg)
+
+
+@pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8), 3 | (67 << 8), 3 | (72 << 8), 3 | (73 << 8)))
 def test_bf16_prefill_large_tiles(flags):
-    # default choice for a large batch, and the two largest tiles forced
+    # default choice for a large batch, and the ring and largest tiles forced
     n, k, m, b, g = 2048, 1024, 2048, 4, 128
     q, s16, z16 = o.make_layer(n, k, g, seed=77)
     s = o.round_to_bf16(s16.astype(np.float32))

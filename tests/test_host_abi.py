@@ -157,14 +157,21 @@ def test_describe_plan_regimes():
 def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     # 640 tiles of 128 x 256 are one round of 512 resident workgroups and a quarter: the rows of
     # the quarter go to narrower tiles; whole rounds, or more than half a round left over, keep the
-    # plain tile; bf16 storage has no such kernel
+    # plain tile
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True).endswith("cfg8")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 57344, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
-    assert not _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3).endswith("cfg8")
-    with pytest.raises(RuntimeError):
-        _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8))
+
+
+def test_planner_gives_bf16_storage_the_narrower_ring_tiles():
+    # bf16 weights are formed in fp32 (twice the vector work per weight): the 128 x 256 tile stalls
+    # on it; 128 x 192 up to 4 bits where its rounds pay, else 128 x 128.  Every tile can be forced.
+    assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3).endswith("cfg9")
+    assert _lib.describe_plan(4, 128, 57344, 8192, 2048, False, 3).endswith("cfg9")
+    assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 3).endswith("cfg3")
+    assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True, 3).endswith("cfg3")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8)).endswith("cfg8")
 
 
 def test_planner_keeps_six_bit_codes_off_the_largest_ring_tile():
