@@ -25,8 +25,8 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
                                 bool stream_flavour, size_t smem, hipStream_t);                \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);          \
   hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, hipStream_t);   \
-  hipError_t launch_gemv_b##B(const GemmArgs&, int shape, int W, size_t lds_pad, bool master, hipStream_t);  \
-  hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int shape, int W, size_t lds_pad, bool master, hipStream_t); \
+  hipError_t launch_gemv_b##B(const GemmArgs&, int group_size, int shape, int W, size_t lds_pad, bool master, hipStream_t);  \
+  hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int group_size, int shape, int W, size_t lds_pad, bool master, hipStream_t); \
   hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, hipStream_t); \
   hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
                                        int kc, bool stream_flavour, size_t smem, hipStream_t); \
@@ -197,16 +197,21 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     p->mb = 1;
     R = mid_rows(1);
   }
-  // Batch rows 1..4 at group size 128: the gemv kernel (every wave requests a whole round of
+  // Batch rows 1..4: the gemv kernel (every wave requests a whole round of
   // tiles at once).  Measured on MI355X (Llama-3-8B layers, every bitwidth): four tiles per
   // wave and round; one row block per workgroup at batch 1 and on layers with few row blocks,
   // two above that (the staged activations of several batch rows are then shared); as many
-  // waves as there are rounds of four tiles, sixteen at most.
-  if (M <= kGemvMaxM && group_size == 128 && flavour == 0 && (variant == 0 || variant >= 100)) {
-    int shape = (M >= 2 && row_blocks >= 320) ? 2 : 1;
+  // waves as there are rounds of four tiles, sixteen at most.  2-bit tiles are half the bytes
+  // for the same work per tile: with two row blocks per workgroup (one staging of the
+  // activations for both) the 28672 x 4096 layer takes 7.7 instead of 8.4 us; the layers with
+  // few row blocks lose that way (4096 x 14336: 6.4 against 5.0 us).
+  // Group sizes 32 and -1 run the two shapes named here (a scale per octet, or per row).
+  if (M <= kGemvMaxM && flavour == 0 && (variant == 0 || variant >= 100)) {
+    int shape = ((M >= 2 && row_blocks >= 320) || (bits == 2 && group_size == 128 && row_blocks >= 1024)) ? 2 : 1;
     if (variant >= 100) {
       shape = variant - 100;
       if (shape >= kNumGemvShapes) return MATGPTQ_EVARIANT;
+      if (group_size != 128 && shape != 1 && shape != 2) return MATGPTQ_EVARIANT;
     }
     const int T = kGemvShapes[shape][0];
     int Wg = (int)((flags >> MATGPTQ_FLAG_GEMV_WAVES_SHIFT) & 31u);
@@ -317,17 +322,17 @@ hipError_t launch_prefill(int bits, bool bf16, const GemmArgs& a, int g, const P
 }
 
 // master: `a.packed` holds master-resident bit planes
-hipError_t launch_gemv(int bits, bool bf16, const GemmArgs& a, const Plan& p, bool master, hipStream_t s) {
+hipError_t launch_gemv(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, bool master, hipStream_t s) {
 #define MATGPTQ_CASE(B) \
-  case B: return bf16 ? launch_gemv_b##B##_bf16(a, p.shape, p.W, p.pad, master, s) \
-                      : launch_gemv_b##B(a, p.shape, p.W, p.pad, master, s);
+  case B: return bf16 ? launch_gemv_b##B##_bf16(a, g, p.shape, p.W, p.pad, master, s) \
+                      : launch_gemv_b##B(a, g, p.shape, p.W, p.pad, master, s);
   switch (bits) {
     MATGPTQ_CASE(2)
     MATGPTQ_CASE(3)
     MATGPTQ_CASE(4)
     MATGPTQ_CASE(6)
-    default: return bf16 ? launch_gemv_b8_bf16(a, p.shape, p.W, p.pad, master, s)
-                         : launch_gemv_b8(a, p.shape, p.W, p.pad, master, s);
+    default: return bf16 ? launch_gemv_b8_bf16(a, g, p.shape, p.W, p.pad, master, s)
+                         : launch_gemv_b8(a, g, p.shape, p.W, p.pad, master, s);
   }
 #undef MATGPTQ_CASE
 }
@@ -400,7 +405,7 @@ static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t 
   a.row_blocks = (int)(N / 16);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
-  const hipError_t err = p.gemv     ? launch_gemv(bitwidth, bf16, a, p, master_planes, s)
+  const hipError_t err = p.gemv     ? launch_gemv(bitwidth, bf16, a, group_size, p, master_planes, s)
                          : p.decode ? launch_decode(bitwidth, bf16, a, group_size, p, s)
                          : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, s)
                                     : launch_prefill(bitwidth, bf16, a, group_size, p, s);
@@ -426,7 +431,8 @@ static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t 
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zp, flags, &p)) return e;
-  *direct = p.gemv && (p.shape == 1 || p.shape == 2);
+  // (the gemv kernel reads the planes directly at group size 128)
+  *direct = p.gemv && group_size == 128 && (p.shape == 1 || p.shape == 2);
   return MATGPTQ_OK;
 }
 

@@ -1,4 +1,4 @@
-// Batch-1..4 kernel for group size 128: the HBM-bound end of the decode regime.
+// Batch-1..4 kernel: the HBM-bound end of the decode regime (group sizes 128, 32 and -1).
 // Compiled once per bitwidth with -DMATGPTQ_BITS=b.
 // Role of the reference's gptq_matryoshka_simt
 // (inference_lib/matgptq_cuda/csrc/matgptq_gemm.cu:636-953); the design is its own.
@@ -24,6 +24,13 @@
 //     acc += scale * (D - off - zero / 2^(8-b) * xs)
 // which is  sum_k scale ((c << (8-b)) - zero) x / 2^(8-b)  over the group.  The partial sums
 // of the four lane quarters and the W waves meet in LDS once, at the end.
+//
+// Group size -1 (one scale per weight row) runs the same chain with the one scale in place of
+// the tile's.  Group size 32 has a scale per octet of a tile, so there the four ROW GROUPS of A
+// take turns per OCTET (row 4j + v is live during the MFMA of octet j): the four MFMAs of one
+// tile leave its four octet sums side by side, lane (n, q) holds the scale and zero of octet q
+// (again one 2-byte load per lane, now per tile), and the per-octet sums  off  and  xs  travel
+// through a small table in LDS (a rotate-reduce over the 4 lanes of an octet fills it).
 #include "tile_format.h"
 
 #ifndef MATGPTQ_BITS
@@ -53,18 +60,34 @@ __device__ __forceinline__ float row_sum16(float v) {
   return add_row_ror<1>(v);
 }
 
-// LDS bytes per wave: X' of one round for MB batch rows + a block of zeros
-constexpr int gemv_wave_lds(int t, int mb) { return mb * t * 256 + 256; }
+// v + the other three lanes of its quad
+__device__ __forceinline__ float quad_sum(float v) {
+  int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+  v += __int_as_float(r);
+  r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false);      // quad_perm [2,3,0,1]
+  return v + __int_as_float(r);
+}
+
+// LDS bytes per wave: X' of one round for MB batch rows + a block of zeros (group 32: as long as
+// one batch row's X', so that tile offsets apply to it too) + group 32's table of octet sums
+constexpr int gemv_zero_bytes(int t, int group) { return group == 32 ? t * 256 : 256; }
+constexpr int gemv_wave_lds(int t, int mb, int group) {
+  return mb * t * 256 + gemv_zero_bytes(t, group) + (group == 32 ? mb * t * 32 : 0);
+}
 
 // MASTER: `a.packed` holds master-resident bit planes (master_layout.h); the rounded slice to
 // BITS is formed in registers while the raw pairs are built.
-template <int BITS, bool ZP, int T, int R, int MB, bool MASTER>
+template <int BITS, bool ZP, int GROUP, int T, int R, int MB, bool MASTER>
 __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
   using Fmt = TileFormat<BITS, MASTER>;
+  constexpr bool kPerOctet = GROUP == 32;  // a scale per octet: the row groups of A take turns per octet
+  static_assert(!kPerOctet || T <= 4, "one lane per 16 bytes of the zero block");
   constexpr int TH = (T + 3) / 4;  // groups of four tiles per round
+  constexpr int NS = GROUP == 128 ? TH : GROUP == 32 ? T : 1;  // scale registers per row block
   constexpr float kMul = (float)(1 << (8 - BITS));
   constexpr int kXBytes = MB * T * 256;
-  constexpr int kWaveBytes = gemv_wave_lds(T, MB);
+  constexpr int kZeroBytes = gemv_zero_bytes(T, GROUP);
+  constexpr int kWaveBytes = gemv_wave_lds(T, MB, GROUP);
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x;
@@ -76,7 +99,8 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 
   unsigned char* xw = smem + wave * kWaveBytes;                   // this wave's X' and zeros
   float* red = reinterpret_cast<float*>(smem + W * kWaveBytes);   // [W][R * MB][64]
-  if (lane < 16) *reinterpret_cast<uint4*>(xw + kXBytes + lane * 16) = make_uint4(0, 0, 0, 0);
+  if (lane * 16 < kZeroBytes) *reinterpret_cast<uint4*>(xw + kXBytes + lane * 16) = make_uint4(0, 0, 0, 0);
+  float2* const osum = reinterpret_cast<float2*>(xw + kXBytes + kZeroBytes);  // group 32: [MB][T][4] (off, xs)
 
   constexpr uint32_t tile_bytes = Fmt::kTileBytes;
   const typename Fmt::Consts consts;
@@ -108,18 +132,24 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
       for (int h = 0; h < TH; h++)
         xv[m][h] = __builtin_amdgcn_raw_buffer_load_b128(xr, lane * 16, (uint32_t)(kt0 + 4 * h) * 256u, 0);
     }
-    uint16_t sv[R][TH], zv[R][TH];
+    uint16_t sv[R][NS], zv[R][NS];
     uint32_t w[R][T][Fmt::kWords];
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
       const bool rows = rb0 + rr < a.row_blocks;
-      const uint32_t g0 = (uint32_t)(rb0 + rr) * a.k_tiles + kt0;  // first tile = first group
-      const BufRsrc sr = make_rsrc(a.scales, rows ? (g0 + nt) * 32u : 0u);
-      const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, rows ? (g0 + nt) * 32u : 0u);
+      const uint32_t g0 = (uint32_t)(rb0 + rr) * a.k_tiles + kt0;  // first tile of the round
+      // bytes of scales per tile and row block: 32 (one group), 128 (four), none (one per row)
+      constexpr uint32_t kSB = GROUP == 128 ? 32u : 128u;
+      const uint32_t s_end = GROUP == -1 ? (uint32_t)(rb0 + rr + 1) * 32u : (g0 + nt) * kSB;
+      const BufRsrc sr = make_rsrc(a.scales, rows ? s_end : 0u);
+      const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, rows ? s_end : 0u);
 #pragma unroll
-      for (int h = 0; h < TH; h++) {
-        sv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(sr, lane * 2, (g0 + 4 * h) * 32u, 0);
-        if constexpr (ZP) zv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(zr, lane * 2, (g0 + 4 * h) * 32u, 0);
+      for (int h = 0; h < NS; h++) {
+        // lane (n, q): group 128, the scale of row n in tile 4 h + q; group 32, in octet q of tile h
+        const uint32_t lo = GROUP == -1 ? (uint32_t)n * 2u : (uint32_t)lane * 2u;
+        const uint32_t so = GROUP == -1 ? (uint32_t)(rb0 + rr) * 32u : GROUP == 128 ? (g0 + 4 * h) * 32u : (g0 + h) * 128u;
+        sv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(sr, lo, so, 0);
+        if constexpr (ZP) zv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(zr, lo, so, 0);
       }
     }
 #pragma unroll
@@ -165,8 +195,17 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         so = dot2(v.p[3], ones, so);
         if (T >= 4 || 4 * h + q < T)
           *reinterpret_cast<uint4*>(xw + m * T * 256 + h * 1024 + lane * 16) = v.v;
-        xs[m][h] = row_sum16(sx);
-        off[m][h] = 1024.0f * row_sum16(so);
+        if constexpr (kPerOctet) {
+          // sums over the four chunks of an octet; the first lane of the quad files them under
+          // (batch row, tile 4 h + lane / 16, octet chunk / 4)
+          const float2 pair = make_float2(1024.0f * quad_sum(so), quad_sum(sx));
+          if ((lane & 3) == 0 && (T >= 4 || 4 * h + q < T)) osum[(m * T + 4 * h + q) * 4 + (n >> 2)] = pair;
+          xs[m][h] = 0.f;
+          off[m][h] = 0.f;
+        } else {
+          xs[m][h] = row_sum16(sx);
+          off[m][h] = 1024.0f * row_sum16(so);
+        }
       }
     }
 
@@ -177,10 +216,17 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 #pragma unroll
     for (int i = 0; i < T; i++) {
       const int u = i & 3;
-      const unsigned char* ab = (n >> 2) == u ? a_live + i * 256 : a_zero;
       Frag av[4];
+      if constexpr (kPerOctet) {
+        // octet j: row group j live (the zero block is as long as X', so `i * 256` applies to both)
 #pragma unroll
-      for (int j = 0; j < 4; j++) av[j].v = *reinterpret_cast<const uint4*>(ab + j * 64);
+        for (int j = 0; j < 4; j++)
+          av[j].v = *reinterpret_cast<const uint4*>(((n >> 2) == j ? a_live : a_zero) + i * 256 + j * 64);
+      } else {
+        const unsigned char* ab = (n >> 2) == u ? a_live + i * 256 : a_zero;
+#pragma unroll
+        for (int j = 0; j < 4; j++) av[j].v = *reinterpret_cast<const uint4*>(ab + j * 64);
+      }
 #pragma unroll
       for (int rr = 0; rr < R; rr++) {
         Frag bw;
@@ -193,15 +239,28 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         Fmt::template raw<3>(w[rr][i], consts, bw.u);
         d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[3].h, bw.h, d[rr], 0, 0, 0);
       }
-      if (u == 3 || i == T - 1) {
+      if (kPerOctet || u == 3 || i == T - 1) {
         const int h = i >> 2;
+        const int si = GROUP == 128 ? h : GROUP == 32 ? i : 0;
+        float fo[MB], fx[MB];
+#pragma unroll
+        for (int v = 0; v < MB; v++) {
+          if constexpr (kPerOctet) {
+            const float2 pair = osum[(v * T + i) * 4 + q];
+            fo[v] = pair.x;
+            fx[v] = pair.y;
+          } else {
+            fo[v] = off[v][h];
+            fx[v] = xs[v][h];
+          }
+        }
 #pragma unroll
         for (int rr = 0; rr < R; rr++) {
-          const float s = storage_to_float(sv[rr][h]);
+          const float s = storage_to_float(sv[rr][si]);
           float zs = (float)(1 << (BITS - 1));
-          if constexpr (ZP) zs = storage_to_float(zv[rr][h]) * (1.0f / kMul);
+          if constexpr (ZP) zs = storage_to_float(zv[rr][si]) * (1.0f / kMul);
 #pragma unroll
-          for (int v = 0; v < MB; v++) acc[rr][v] += s * (d[rr][v] - off[v][h] - zs * xs[v][h]);
+          for (int v = 0; v < MB; v++) acc[rr][v] += s * (d[rr][v] - fo[v] - zs * fx[v]);
           d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
         }
       }
@@ -226,59 +285,59 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 }
 
 // WPE: waves per SIMD the register allocation is held to
-template <int BITS, bool ZP, int T, int R, int MB, int WPE, bool MASTER>
+template <int BITS, bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER>
 __global__ void __launch_bounds__(1024, WPE) gemv_kernel(const GemmArgs a, const int W) {
-  gemv_body<BITS, ZP, T, R, MB, MASTER>(a, W);
+  gemv_body<BITS, ZP, GROUP, T, R, MB, MASTER>(a, W);
 }
 
-template <bool ZP, int T, int R, int MB, int WPE, bool MASTER>
+template <bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER>
 hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stream) {
   const dim3 grid((a.row_blocks + R - 1) / R), block(64 * W);
-  size_t smem = (size_t)W * gemv_wave_lds(T, MB) + (size_t)W * R * MB * 256;
+  size_t smem = (size_t)W * gemv_wave_lds(T, MB, GROUP) + (size_t)W * R * MB * 256;
   if (smem < lds_pad) smem = lds_pad;
   if (W < 1 || W > 16 || a.M > MB || smem > 160 * 1024) return hipErrorInvalidValue;
   if (smem > 64 * 1024) {
     // more than 64 KiB of dynamic LDS has to be allowed once per kernel
     static bool allowed = false;
     if (!allowed) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, T, R, MB, WPE, MASTER>),
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
       allowed = true;
     }
   }
-  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, T, R, MB, WPE, MASTER>), grid, block, smem, stream, a, W);
+  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER>), grid, block, smem, stream, a, W);
   return hipGetLastError();
 }
 
 // shapes built: (T tiles per wave and round, R row blocks per workgroup); the master-resident
-// storage takes the two shapes the planner uses
-template <bool ZP, int MB, bool MASTER>
+// storage and the group sizes 32 and -1 take the two shapes the planner uses
+template <bool ZP, int GROUP, int MB, bool MASTER>
 hipError_t launch_shape(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t s) {
-  if constexpr (MASTER) {
-    if (shape == 2) return launch_one<ZP, 4, 2, MB, 4, true>(a, W, lds_pad, s);
-    if (shape == 1) return launch_one<ZP, 4, 1, MB, 4, true>(a, W, lds_pad, s);
+  if constexpr (MASTER || GROUP != 128) {
+    if (shape == 2) return launch_one<ZP, GROUP, 4, 2, MB, 4, MASTER>(a, W, lds_pad, s);
+    if (shape == 1) return launch_one<ZP, GROUP, 4, 1, MB, 4, MASTER>(a, W, lds_pad, s);
     return hipErrorInvalidValue;
   } else {
     switch (shape) {
-      case 0: return launch_one<ZP, 8, 1, MB, 4, false>(a, W, lds_pad, s);
-      case 1: return launch_one<ZP, 4, 1, MB, 4, false>(a, W, lds_pad, s);
-      case 2: return launch_one<ZP, 4, 2, MB, 4, false>(a, W, lds_pad, s);
-      case 3: return launch_one<ZP, 2, 2, MB, 4, false>(a, W, lds_pad, s);
-      case 4: return launch_one<ZP, 2, 4, MB, 4, false>(a, W, lds_pad, s);
-      default: return launch_one<ZP, 2, 1, MB, 4, false>(a, W, lds_pad, s);
+      case 0: return launch_one<ZP, 128, 8, 1, MB, 4, false>(a, W, lds_pad, s);
+      case 1: return launch_one<ZP, 128, 4, 1, MB, 4, false>(a, W, lds_pad, s);
+      case 2: return launch_one<ZP, 128, 4, 2, MB, 4, false>(a, W, lds_pad, s);
+      case 3: return launch_one<ZP, 128, 2, 2, MB, 4, false>(a, W, lds_pad, s);
+      case 4: return launch_one<ZP, 128, 2, 4, MB, 4, false>(a, W, lds_pad, s);
+      default: return launch_one<ZP, 128, 2, 1, MB, 4, false>(a, W, lds_pad, s);
     }
   }
 }
 
-template <bool MASTER>
+template <int GROUP, bool MASTER>
 hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t stream) {
   const bool zp = a.zeros != nullptr;
   if (a.M == 1)
-    return zp ? launch_shape<true, 1, MASTER>(a, shape, W, lds_pad, stream)
-              : launch_shape<false, 1, MASTER>(a, shape, W, lds_pad, stream);
-  return zp ? launch_shape<true, 4, MASTER>(a, shape, W, lds_pad, stream)
-            : launch_shape<false, 4, MASTER>(a, shape, W, lds_pad, stream);
+    return zp ? launch_shape<true, GROUP, 1, MASTER>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, GROUP, 1, MASTER>(a, shape, W, lds_pad, stream);
+  return zp ? launch_shape<true, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream)
+            : launch_shape<false, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream);
 }
 
 }  // namespace
@@ -286,7 +345,7 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 // Entry of this translation unit.  shape: index into the (T, R) table above; W: waves per
 // workgroup (1..16); lds_pad: dynamic LDS to ask for when it exceeds what the kernel needs
 // (limits how many workgroups share a CU); master: `a.packed` holds master-resident bit planes
-// (shapes 1 and 2 only).  Group size 128 and M <= 4 only.
+// (shapes 1 and 2, group size 128 only); group sizes 32 and -1: shapes 1 and 2.  M <= 4 only.
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 #if MATGPTQ_BF16
@@ -294,10 +353,12 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 #else
 #define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_gemv_b, MATGPTQ_BITS)
 #endif
-hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int shape, int W, size_t lds_pad, bool master,
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int shape, int W, size_t lds_pad, bool master,
                                hipStream_t stream) {
-  return master ? launch_storage<true>(a, shape, W, lds_pad, stream)
-                : launch_storage<false>(a, shape, W, lds_pad, stream);
+  if (group_size == 32) return master ? hipErrorInvalidValue : launch_storage<32, false>(a, shape, W, lds_pad, stream);
+  if (group_size == -1) return master ? hipErrorInvalidValue : launch_storage<-1, false>(a, shape, W, lds_pad, stream);
+  return master ? launch_storage<128, true>(a, shape, W, lds_pad, stream)
+                : launch_storage<128, false>(a, shape, W, lds_pad, stream);
 }
 
 }  // namespace matgptq

@@ -1,7 +1,8 @@
-"""The batch-1..4 kernel for group size 128 (gemv_gfx950.hip) against the oracle, through the C ABI.
+"""The batch-1..4 kernel (gemv_gfx950.hip) against the oracle, through the C ABI.
 
 Every instantiation (tiles per wave and round x row blocks per workgroup), every bitwidth,
-both zero-point forms, ragged row-block counts and ragged rounds of K tiles, both storage types.
+both zero-point forms, ragged row-block counts and ragged rounds of K tiles, both storage types,
+the three group sizes.
 """
 import numpy as np
 import pytest
@@ -38,11 +39,63 @@ def test_gemv_every_instantiation(b, zp):
                 G.assert_regression_bound(y, x, lay.w, f"b={b} zp={zp} M={m} shape={shape} W={waves}")
 
 
+@pytest.mark.parametrize("g", (32, -1))
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("b", BITS)
+def test_gemv_group_sizes_32_and_per_row(b, zp, g):
+    # a scale per octet of a tile (the row groups of the activation operand take turns per octet)
+    # and a scale per weight row; ragged row blocks and rounds as above
+    n, k = 80, 128 * 13
+    lay = G.Layer(n, k, b, g, seed=60 + b, zero_points=zp)
+    for m in (1, 2, 3, 4):
+        x = o.make_activations(m, k, seed=m + b, outlier_frac=0.01)
+        assert _lib.describe_plan(b, g, n, k, m, zp).startswith("gemv")
+        G.assert_close_to_oracle(lay.run(x), x, lay.w, f"default b={b} g={g} zp={zp} M={m}")
+        for shape in (1, 2):
+            for waves in (0, 1, 3, 16):
+                y = lay.run(x, flags=gemv_flags(shape, waves))
+                G.assert_close_to_oracle(y, x, lay.w, f"b={b} g={g} zp={zp} M={m} shape={shape} W={waves}")
+                G.assert_regression_bound(y, x, lay.w, f"b={b} g={g} zp={zp} M={m} shape={shape} W={waves}")
+
+
+@pytest.mark.parametrize("g", (32, -1))
+def test_gemv_group_sizes_exact_in_the_reference_test_regime(g):
+    # 0/1 scales, integer activations, symmetric form: the closed form, bit for bit
+    rng = np.random.default_rng(6)
+    n, k = 48, 4096
+    G_ = 1 if g == -1 else k // g
+    for b in BITS:
+        codes = rng.integers(0, 1 << b, (n, k), dtype=np.uint8)
+        scales = np.round(rng.random((n, G_))).astype(np.float16)
+        if g == -1:
+            scales[:] = 1.0  # (a row of 4096 columns at scale 0 would test nothing)
+        pk = G.pack_device(codes, b, from_master=False)
+        sd = G.reorder_device(scales, n, k, g)
+        w = o.dequantize_kernel_form(codes, scales, b, g)
+        for m in (1, 4):
+            x = np.round(rng.standard_normal((m, k))).astype(np.float16)
+            expect = o.linear_f64(x, w).astype(np.float16)
+            for shape in (1, 2):
+                y = G.gemm(b, g, n, k, G.to_dev(x), pk, sd, None, flags=gemv_flags(shape)).cpu().numpy()
+                assert np.array_equal(y.view(np.uint16), expect.view(np.uint16)), (b, g, m, shape)
+
+
+def test_gemv_group_sizes_agree_with_the_decode_kernel():
+    n, k, b = 1024, 4096, 4
+    for g in (32, -1):
+        lay = G.Layer(n, k, b, g, seed=11)
+        for m in (1, 3):
+            x = o.make_activations(m, k, seed=m)
+            a = lay.run(x).astype(np.float64)
+            c = lay.run(x, flags=1 | (1 << 16)).astype(np.float64)  # burst flavour: the decode kernel
+            assert _lib.describe_plan(b, g, n, k, m, True, 1 | (1 << 16)).startswith("decode")
+            assert np.max(np.abs(a - c)) <= 2.0 ** -9 * np.max(np.abs(c))
+
+
 def test_gemv_is_not_taken_outside_its_domain():
     assert _lib.describe_plan(4, 128, 4096, 4096, 5, True).split()[0] in ("decode-burst", "midbatch")
-    assert _lib.describe_plan(4, 32, 4096, 4096, 1, True).startswith("decode")
-    assert _lib.describe_plan(4, -1, 4096, 4096, 1, True).startswith("decode")
-    with pytest.raises(_lib.MatGPTQError, match="variant"):
+    assert _lib.describe_plan(4, 32, 4096, 4096, 5, True).split()[0].startswith(("decode", "midbatch"))
+    with pytest.raises(_lib.MatGPTQError, match="variant"):  # group 32: shapes 1 and 2 only
         G.Layer(32, 256, 4, 32, seed=1).run(o.make_activations(1, 256, seed=1), flags=gemv_flags(0))
     with pytest.raises(_lib.MatGPTQError, match="variant"):
         G.Layer(32, 256, 4, 128, seed=1).run(o.make_activations(5, 256, seed=1), flags=gemv_flags(0))

@@ -126,14 +126,16 @@ def test_error_codes():
 
 
 def test_describe_plan_regimes():
-    # batch 1..4 at group 128: the gemv kernel; other groups and five rows on: decode / mid-batch
+    # batch 1..4: the gemv kernel; five rows on: decode / mid-batch
     assert _lib.describe_plan(4, 128, 4096, 4096, 1) == "gemv b4 g128 zp0 T4 R1 W8 pad0"
     assert _lib.describe_plan(4, 128, 4096, 14336, 1, True) == "gemv b4 g128 zp1 T4 R1 W16 pad0"
     assert _lib.describe_plan(4, 128, 4096, 4096, 4, True) == "gemv b4 g128 zp1 T4 R1 W8 pad0"
     assert _lib.describe_plan(4, 128, 28672, 4096, 4, True) == "gemv b4 g128 zp1 T4 R2 W8 pad0"
     assert _lib.describe_plan(4, 128, 4096, 4096, 1, True, 1 | (1 << 16)).startswith("decode-burst")
-    assert _lib.describe_plan(4, 32, 4096, 4096, 1).startswith("decode")
-    assert _lib.describe_plan(4, -1, 4096, 4096, 4).startswith("decode")
+    assert _lib.describe_plan(4, 32, 4096, 4096, 1) == "gemv b4 g32 zp0 T4 R1 W8 pad0"
+    assert _lib.describe_plan(4, -1, 4096, 4096, 4) == "gemv b4 g-1 zp0 T4 R1 W8 pad0"
+    assert _lib.describe_plan(2, 128, 28672, 4096, 1, True) == "gemv b2 g128 zp1 T4 R2 W8 pad0"
+    assert _lib.describe_plan(4, 32, 4096, 4096, 5).startswith(("decode", "midbatch"))
     assert _lib.describe_plan(4, 128, 28672, 4096, 5, True).startswith("decode")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048).startswith("prefill")
     with pytest.raises(RuntimeError):
@@ -146,7 +148,7 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(4, 128, 28672, 4096, 16, True) == "midbatch b4 g128 zp1 R4 mb1"
     # small layers: the mid-batch kernel (K split inside the workgroup) from a few rows on
     assert _lib.describe_plan(4, 128, 4096, 4096, 8, True).startswith("midbatch")
-    assert _lib.describe_plan(4, 32, 4096, 14336, 2, True).startswith("midbatch")
+    assert _lib.describe_plan(4, 32, 4096, 14336, 5, True).startswith("midbatch")
     assert _lib.describe_plan(3, 32, 16, 1024, 17).startswith("midbatch")
     assert _lib.describe_plan(4, 128, 4096, 4096, 128, True) == "midbatch b4 g128 zp1 R4 mb2"
     assert _lib.describe_plan(8, 128, 4096, 4096, 128, True) == "midbatch b8 g128 zp1 R2 mb2"
