@@ -11,7 +11,9 @@
  * Y = X * W^T is [M, N].  The reference calls them m (=N), n (=K), k (=M).
  *
  * Preconditions shared by all entry points: bitwidth in {2,3,4,6,8},
- * group_size in {-1,32,128}, N % 16 == 0, K % 128 == 0.
+ * group_size in {-1,32,128}, N % 16 == 0, K % 128 == 0 or (group sizes 32 and -1) K % 128 == 64
+ * with K >= 192 (the reference: K % 64 == 0, inference_lib/matgptq_cuda/csrc/utils.cpp:174-184);
+ * the master-resident entry points take K % 128 == 0 only.
  */
 #ifndef MATGPTQ_ABI_H
 #define MATGPTQ_ABI_H
@@ -29,7 +31,7 @@ extern "C" {
 #define MATGPTQ_OK 0
 #define MATGPTQ_EBITS (-1)     /* bitwidth not in {2,3,4,6,8} */
 #define MATGPTQ_EGROUP (-2)    /* group_size not in {-1,32,128} or does not divide K */
-#define MATGPTQ_ESHAPE (-3)    /* N % 16 != 0, K % 128 != 0, or a size <= 0 */
+#define MATGPTQ_ESHAPE (-3)    /* N % 16 != 0, K not of the forms above, or a size <= 0 */
 #define MATGPTQ_ENULL (-4)     /* a required pointer is NULL */
 #define MATGPTQ_EDTYPE (-5)    /* operation not available for the requested data type */
 #define MATGPTQ_ELAUNCH (-6)   /* the HIP runtime reported an error at launch */

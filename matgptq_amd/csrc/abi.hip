@@ -44,6 +44,7 @@ hipError_t launch_slice(const uint8_t*, int64_t, int, uint8_t*, hipStream_t);
 hipError_t launch_pack_master(const uint8_t*, int64_t, int64_t, uint32_t*, hipStream_t);
 hipError_t launch_master_slice(const uint32_t*, int64_t, int64_t, int, bool, void*, hipStream_t);
 hipError_t launch_reorder(const uint16_t*, int64_t, int64_t, uint16_t*, hipStream_t);
+hipError_t launch_tail_gemm(int bits, bool bf16, const GemmArgs&, int group_size, hipStream_t);
 hipError_t launch_dequant(int, int, int64_t, int64_t, const uint32_t*, const uint16_t*,
                           const uint16_t*, uint16_t*, hipStream_t);
 
@@ -364,7 +365,9 @@ const char* matgptq_strerror(int code) {
     case MATGPTQ_OK: return "ok";
     case MATGPTQ_EBITS: return "bitwidth must be one of {2, 3, 4, 6, 8}";
     case MATGPTQ_EGROUP: return "group_size must be one of {-1, 32, 128} and divide n_in_features";
-    case MATGPTQ_ESHAPE: return "n_out_features must be a multiple of 16 and n_in_features a multiple of 128";
+    case MATGPTQ_ESHAPE:
+      return "n_out_features must be a multiple of 16 and n_in_features a multiple of 128 (or, at group sizes 32 and -1, "
+             "such a multiple plus 64; master-resident planes: a multiple of 128)";
     case MATGPTQ_ENULL: return "null pointer argument";
     case MATGPTQ_EDTYPE: return "unsupported data type for this operation (float16 only)";
     case MATGPTQ_ELAUNCH: return "HIP launch failed";
@@ -410,6 +413,8 @@ static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t 
                          : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, s)
                                     : launch_prefill(bitwidth, bf16, a, group_size, p, s);
   if (err != hipSuccess) return MATGPTQ_ELAUNCH;
+  // K = 128 t + 64: the kernels above have multiplied the t tiles; a second launch adds the last 64 columns
+  if (K % 128 != 0 && launch_tail_gemm(bitwidth, bf16, a, group_size, s) != hipSuccess) return MATGPTQ_ELAUNCH;
   if (!(flags & MATGPTQ_FLAG_ASYNC)) {
     if (hipStreamSynchronize(s) != hipSuccess) return MATGPTQ_ELAUNCH;
   }
@@ -428,6 +433,7 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
 static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M, bool zp,
                                uint32_t flags, bool* direct) {
   if (int e = check_problem(bitwidth, group_size, N, K)) return e;
+  if (K % 128 != 0) return MATGPTQ_ESHAPE;  // the bit planes have whole tiles only
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zp, flags, &p)) return e;
@@ -508,6 +514,7 @@ int matgptq_gemm_master_static(int bitwidth, int group_size, int64_t N, int64_t 
 int matgptq_pack_master_device(const uint8_t* codes_dev, int64_t N, int64_t K, uint32_t* planes_dev,
                                void* stream) {
   if (int e = check_problem(8, -1, N, K)) return e;
+  if (K % 128 != 0) return MATGPTQ_ESHAPE;
   if (!codes_dev || !planes_dev) return MATGPTQ_ENULL;
   return launch_pack_master(codes_dev, N, K, planes_dev, static_cast<hipStream_t>(stream)) == hipSuccess
              ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
@@ -516,6 +523,7 @@ int matgptq_pack_master_device(const uint8_t* codes_dev, int64_t N, int64_t K, u
 int matgptq_unpack_master_device(const uint32_t* planes_dev, int64_t N, int64_t K, int bitwidth,
                                  uint8_t* codes_dev, void* stream) {
   if (int e = check_problem(bitwidth, -1, N, K)) return e;
+  if (K % 128 != 0) return MATGPTQ_ESHAPE;
   if (!planes_dev || !codes_dev) return MATGPTQ_ENULL;
   return launch_master_slice(planes_dev, N, K, bitwidth, false, codes_dev, static_cast<hipStream_t>(stream)) ==
                  hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;

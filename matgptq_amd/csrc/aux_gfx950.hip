@@ -214,9 +214,144 @@ master_slice_kernel(const uint32_t* __restrict__ planes, void* __restrict__ out,
   }
 }
 
+// ---- the tail of K = 128 t + 64 (layout.h): 64 columns per row as a bitstream ---------------
+// one thread = one row
+__global__ void __launch_bounds__(256)
+pack_tail_kernel(const uint8_t* __restrict__ codes, uint32_t* __restrict__ tail, int64_t N, int64_t K,
+                 int bits, int slice) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  const uint8_t* src = codes + n * K + (K - kTailCols);
+  uint8_t c[kTailCols];
+  for (int k = 0; k < kTailCols; k++) c[k] = slice ? slice_code(src[k], bits) : src[k];
+  uint32_t row[16];
+  tail_encode_row(c, bits, row);
+  for (int i = 0; i < tail_row_words(bits); i++) tail[n * tail_row_words(bits) + i] = row[i];
+}
+
+// one thread = one code
+__global__ void __launch_bounds__(256)
+unpack_tail_kernel(const uint32_t* __restrict__ tail, uint8_t* __restrict__ codes, int64_t N, int64_t K, int bits) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * kTailCols) return;
+  const int64_t n = i / kTailCols;
+  const int k = (int)(i - n * kTailCols);
+  codes[n * K + (K - kTailCols) + k] = (uint8_t)tail_code(tail + n * tail_row_words(bits), bits, k);
+}
+
+// scale and zero of (row n, column k) from the reordered [N/16][G][16] tensors, as float
+template <bool BF16>
+__device__ __forceinline__ void tail_scale_zero(const uint16_t* scales, const uint16_t* zeros, int64_t n, int64_t k,
+                                                int G, int group_size, float& s, float& z) {
+  const int64_t g = group_size == -1 ? 0 : k / group_size;
+  const size_t so = ((size_t)(n >> 4) * G + g) * 16 + (n & 15);
+  if constexpr (BF16) {
+    s = bf16_bits_to_float(scales[so]);
+    z = zeros ? bf16_bits_to_float(zeros[so]) : 128.0f;
+  } else {
+    s = (float)__builtin_bit_cast(_Float16, scales[so]);
+    z = zeros ? (float)__builtin_bit_cast(_Float16, zeros[so]) : 128.0f;
+  }
+}
+
+// one weight the way dequantize() forms it on tensors of the storage type: the difference and the
+// product are each rounded to that type
+template <bool BF16>
+__device__ __forceinline__ float tail_weight(uint32_t code, int bits, float s, float z) {
+  const float d = (float)(int)(code << (8 - bits)) - z;
+  if constexpr (BF16) {
+    const float dr = bf16_bits_to_float(float_to_bf16_bits(d));
+    return bf16_bits_to_float(float_to_bf16_bits(s * dr));
+  } else {
+    const float dr = (float)(_Float16)d;
+    return (float)(_Float16)(s * dr);
+  }
+}
+
+// dense dequantise, tail columns: one thread = one weight (fp16 storage, like dequant_kernel)
+__global__ void __launch_bounds__(256)
+dequant_tail_kernel(const uint32_t* __restrict__ tail, const uint16_t* __restrict__ scales,
+                    const uint16_t* __restrict__ zeros, uint16_t* __restrict__ w_out, int64_t N, int64_t K,
+                    int G, int group_size, int bits) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * kTailCols) return;
+  const int64_t n = i / kTailCols;
+  const int64_t k = (K - kTailCols) + (i - n * kTailCols);
+  float s, z;
+  tail_scale_zero<false>(scales, zeros, n, k, G, group_size, s, z);
+  const float w = tail_weight<false>(tail_code(tail + n * tail_row_words(bits), bits, (int)(i - n * kTailCols)), bits, s, z);
+  w_out[n * K + k] = __builtin_bit_cast(uint16_t, (_Float16)w);
+}
+
+// Y[m][n] += sum over the tail columns of X[m][k] W[n][k]: runs after the GEMM over the tiles has
+// written Y.  A workgroup = 16 weight rows x 16 lanes of batch rows; a thread keeps the 64 weights
+// of its row in registers and walks `m_per_block` / 16 batch rows.  N x 64 weights against a GEMM of
+// N x 128 t: a plain vector-ALU kernel is enough.
+template <bool BF16>
+__global__ void __launch_bounds__(256)
+tail_gemm_kernel(const uint32_t* __restrict__ tail, const uint16_t* __restrict__ scales,
+                 const uint16_t* __restrict__ zeros, const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                 int N, int K, int M, int G, int group_size, int bits, int m_per_block) {
+  const int n = blockIdx.x * 16 + (threadIdx.x & 15);
+  const int ml = threadIdx.x >> 4;
+  const int K0 = K - kTailCols;
+  const uint32_t* row = tail + (size_t)n * tail_row_words(bits);
+  float w[kTailCols];
+#pragma unroll
+  for (int k8 = 0; k8 < kTailCols / 32; k8++) {  // a scale per 32 columns at most
+    float s, z;
+    tail_scale_zero<BF16>(scales, zeros, n, K0 + k8 * 32, G, group_size, s, z);
+#pragma unroll
+    for (int k = 0; k < 32; k++) w[k8 * 32 + k] = tail_weight<BF16>(tail_code(row, bits, k8 * 32 + k), bits, s, z);
+  }
+  const int m_end = min(M, (int)(blockIdx.y + 1) * m_per_block);
+  for (int m = blockIdx.y * m_per_block + ml; m < m_end; m += 16) {
+    const uint4* xp = reinterpret_cast<const uint4*>(x + (size_t)m * K + K0);
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < kTailCols / 8; c++) {
+      const uint4 v = xp[c];
+      const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float lo, hi;
+        if constexpr (BF16) {
+          lo = bf16_bits_to_float(u[e] & 0xffffu);
+          hi = bf16_bits_to_float(u[e] >> 16);
+        } else {
+          lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[e] & 0xffffu));
+          hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(u[e] >> 16));
+        }
+        acc = __builtin_fmaf(lo, w[c * 8 + 2 * e], acc);
+        acc = __builtin_fmaf(hi, w[c * 8 + 2 * e + 1], acc);
+      }
+    }
+    uint16_t* yp = y + (size_t)m * N + n;
+    if constexpr (BF16) *yp = (uint16_t)float_to_bf16_bits(bf16_bits_to_float(*yp) + acc);
+    else *yp = __builtin_bit_cast(uint16_t, (_Float16)((float)__builtin_bit_cast(_Float16, *yp) + acc));
+  }
+}
+
 inline unsigned blocks_for(int64_t n, int per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
+// first word of the tail: behind the tiles of all row blocks
+inline int64_t tail_offset_words(int64_t N, int64_t K, int bits) { return (N / 16) * (K / 128) * tile_words(bits); }
+
 }  // namespace
+
+// Adds the product over the last 64 columns (K = 128 t + 64) to Y; `a` as for the GEMM kernels.
+hipError_t launch_tail_gemm(int bits, bool bf16, const GemmArgs& a, int group_size, hipStream_t s) {
+  const uint32_t* tail = a.packed + tail_offset_words(a.N, a.K, bits);
+  const int m_per_block = 128;
+  const dim3 grid(a.N / 16, (a.M + m_per_block - 1) / m_per_block), block(256);
+  if (bf16)
+    hipLaunchKernelGGL(tail_gemm_kernel<true>, grid, block, 0, s, tail, a.scales, a.zeros, a.x, a.y, a.N, a.K, a.M, a.G,
+                       group_size, bits, m_per_block);
+  else
+    hipLaunchKernelGGL(tail_gemm_kernel<false>, grid, block, 0, s, tail, a.scales, a.zeros, a.x, a.y, a.N, a.K, a.M, a.G,
+                       group_size, bits, m_per_block);
+  return hipGetLastError();
+}
 
 hipError_t launch_pack(const uint8_t* codes, int64_t N, int64_t K, int bits, int slice,
                        uint32_t* out, hipStream_t s) {
@@ -230,6 +365,9 @@ hipError_t launch_pack(const uint8_t* codes, int64_t N, int64_t K, int bits, int
     case 6: hipLaunchKernelGGL(pack_kernel<6>, grid, block, 0, s, codes, out, k_tiles, K, slots, slice); break;
     default: hipLaunchKernelGGL(pack_kernel<8>, grid, block, 0, s, codes, out, k_tiles, K, slots, slice); break;
   }
+  if (K % 128 != 0)
+    hipLaunchKernelGGL(pack_tail_kernel, dim3(blocks_for(N, 256)), block, 0, s, codes, out + tail_offset_words(N, K, bits),
+                       N, K, bits, slice);
   return hipGetLastError();
 }
 
@@ -245,6 +383,9 @@ hipError_t launch_unpack(const uint32_t* packed, int64_t N, int64_t K, int bits,
     case 6: hipLaunchKernelGGL(unpack_kernel<6>, grid, block, 0, s, packed, codes, k_tiles, K, slots); break;
     default: hipLaunchKernelGGL(unpack_kernel<8>, grid, block, 0, s, packed, codes, k_tiles, K, slots); break;
   }
+  if (K % 128 != 0)
+    hipLaunchKernelGGL(unpack_tail_kernel, dim3(blocks_for(N * kTailCols, 256)), block, 0, s,
+                       packed + tail_offset_words(N, K, bits), codes, N, K, bits);
   return hipGetLastError();
 }
 
@@ -309,6 +450,9 @@ hipError_t launch_dequant(int bits, int group_size, int64_t N, int64_t K, const 
     default: MATGPTQ_DQ(8); break;
   }
 #undef MATGPTQ_DQ
+  if (K % 128 != 0)
+    hipLaunchKernelGGL(dequant_tail_kernel, dim3(blocks_for(N * kTailCols, 256)), block, 0, s,
+                       packed + tail_offset_words(N, K, bits), scales, zeros, w, N, K, G, group_size, bits);
   return hipGetLastError();
 }
 

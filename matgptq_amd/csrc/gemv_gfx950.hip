@@ -138,16 +138,18 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
     for (int rr = 0; rr < R; rr++) {
       const bool rows = rb0 + rr < a.row_blocks;
       const uint32_t g0 = (uint32_t)(rb0 + rr) * a.k_tiles + kt0;  // first tile of the round
-      // bytes of scales per tile and row block: 32 (one group), 128 (four), none (one per row)
+      // scales of a row block: G groups of 16 values; a tile spans one group (32 bytes), or four at
+      // group size 32 (G may then be 4 K/128 + 2: the last 64 columns are not this kernel's)
+      const uint32_t sg0 = (uint32_t)(rb0 + rr) * a.G + (GROUP == 32 ? 4u : 1u) * kt0;  // first group of the round
       constexpr uint32_t kSB = GROUP == 128 ? 32u : 128u;
-      const uint32_t s_end = GROUP == -1 ? (uint32_t)(rb0 + rr + 1) * 32u : (g0 + nt) * kSB;
+      const uint32_t s_end = GROUP == -1 ? (uint32_t)(rb0 + rr + 1) * 32u : sg0 * 32u + nt * kSB;
       const BufRsrc sr = make_rsrc(a.scales, rows ? s_end : 0u);
       const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, rows ? s_end : 0u);
 #pragma unroll
       for (int h = 0; h < NS; h++) {
         // lane (n, q): group 128, the scale of row n in tile 4 h + q; group 32, in octet q of tile h
         const uint32_t lo = GROUP == -1 ? (uint32_t)n * 2u : (uint32_t)lane * 2u;
-        const uint32_t so = GROUP == -1 ? (uint32_t)(rb0 + rr) * 32u : GROUP == 128 ? (g0 + 4 * h) * 32u : (g0 + h) * 128u;
+        const uint32_t so = GROUP == -1 ? (uint32_t)(rb0 + rr) * 32u : (sg0 + 4 * h) * 32u;  // (group 32: h = tile)
         sv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(sr, lo, so, 0);
         if constexpr (ZP) zv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(zr, lo, so, 0);
       }

@@ -27,6 +27,11 @@
 // (inference_lib/matgptq_cuda/csrc/bindings.cpp:68,160); the byte order inside
 // is private, as it is in the reference.
 //
+// K = 128 t + 64 (group sizes 32 and -1 only; the reference packs any K % 64 == 0,
+// inference_lib/matgptq_cuda/csrc/utils.cpp:174-184): the t tiles of every row block come first,
+// as above with K/128 = t; the last 64 columns of all rows (the TAIL) follow them as plain
+// bitstreams, 2 b words per row, code k of a row at bit k * b.  Still b*N*K/32 words.
+//
 // Inside a word the fields are permuted so that a mask, an OR with 0x6400 and
 // at most one shift leave two codes as the low mantissa bits of a packed pair
 // of fp16 numbers 1024 + c * 2^p.  `decode_octet` below produces these "raw"
@@ -51,6 +56,29 @@ constexpr uint32_t kMagic = 0x64006400u;  // two fp16 1024.0
 constexpr bool valid_bits(int b) { return b == 2 || b == 3 || b == 4 || b == 6 || b == 8; }
 constexpr bool valid_group(int g) { return g == -1 || g == 32 || g == 128; }
 constexpr int tile_words(int b) { return 64 * b; }
+
+// The tail of K = 128 t + 64.
+constexpr int kTailCols = 64;
+constexpr int tail_row_words(int b) { return 2 * b; }
+// K is a multiple of 128, or such a multiple (at least one tile) plus 64
+constexpr bool valid_k(int64_t K) { return K > 0 && (K % 128 == 0 || (K % 128 == 64 && K >= 192)); }
+// code k (0..63) of a tail row stored at `row` (2 b words)
+MATGPTQ_HD uint32_t tail_code(const uint32_t* row, int b, int k) {
+  const int bit = k * b, w = bit >> 5, sh = bit & 31;
+  uint32_t v = row[w] >> sh;
+  if (sh + b > 32) v |= row[w + 1] << (32 - sh);
+  return v & ((1u << b) - 1u);
+}
+// 64 codes -> the 2 b words of a tail row
+MATGPTQ_HD void tail_encode_row(const uint8_t* codes, int b, uint32_t* row) {
+  for (int i = 0; i < 2 * b; i++) row[i] = 0u;
+  for (int k = 0; k < kTailCols; k++) {
+    const uint32_t c = (uint32_t)codes[k] & ((1u << b) - 1u);
+    const int bit = k * b, w = bit >> 5, sh = bit & 31;
+    row[w] |= c << sh;
+    if (sh + b > 32) row[w + 1] |= c >> (32 - sh);
+  }
+}
 
 // Number of words of the first segment per lane; the second segment (if any)
 // holds the remaining words.

@@ -12,7 +12,7 @@ namespace matgptq {
 
 int check_problem(int bits, int group_size, int64_t N, int64_t K) {
   if (!valid_bits(bits)) return MATGPTQ_EBITS;
-  if (N <= 0 || K <= 0 || N % kTileRows != 0 || K % kTileCols != 0) return MATGPTQ_ESHAPE;
+  if (N <= 0 || N % kTileRows != 0 || !valid_k(K)) return MATGPTQ_ESHAPE;
   if (!valid_group(group_size)) return MATGPTQ_EGROUP;
   if (group_size != -1 && K % group_size != 0) return MATGPTQ_EGROUP;
   return MATGPTQ_OK;
@@ -40,6 +40,18 @@ static void pack_impl(const uint8_t* codes, int64_t N, int64_t K, bool slice, ui
       }
     }
   }
+  if (K % kTileCols != 0) {  // the last 64 columns, one bitstream per row
+    uint32_t* tail = out + row_blocks * k_blocks * tile_words(BITS);
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+      uint8_t c[kTailCols];
+      for (int k = 0; k < kTailCols; k++) {
+        const uint8_t v = codes[n * K + k_blocks * kTileCols + k];
+        c[k] = slice ? slice_code(v, BITS) : v;
+      }
+      tail_encode_row(c, BITS, tail + n * tail_row_words(BITS));
+    }
+  }
 }
 
 template <int BITS>
@@ -61,6 +73,13 @@ static void unpack_impl(const uint32_t* packed, int64_t N, int64_t K, uint8_t* c
         }
       }
     }
+  }
+  if (K % kTileCols != 0) {
+    const uint32_t* tail = packed + row_blocks * k_blocks * tile_words(BITS);
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++)
+      for (int k = 0; k < kTailCols; k++)
+        codes[n * K + k_blocks * kTileCols + k] = (uint8_t)tail_code(tail + n * tail_row_words(BITS), BITS, k);
   }
 }
 
@@ -131,6 +150,7 @@ size_t matgptq_master_words(int64_t N, int64_t K) {
 
 int matgptq_pack_master_host(const uint8_t* codes_host, int64_t N, int64_t K, uint32_t* out_host) {
   if (int e = check_problem(8, -1, N, K)) return e;
+  if (K % kTileCols != 0) return MATGPTQ_ESHAPE;  // the bit planes have whole tiles only
   if (!codes_host || !out_host) return MATGPTQ_ENULL;
   const int64_t row_blocks = N / kTileRows, k_blocks = K / kTileCols;
 #pragma omp parallel for schedule(static)
@@ -153,6 +173,7 @@ int matgptq_pack_master_host(const uint8_t* codes_host, int64_t N, int64_t K, ui
 int matgptq_unpack_master_host(const uint32_t* planes_host, int64_t N, int64_t K, int bitwidth,
                                uint8_t* codes_host) {
   if (int e = check_problem(bitwidth, -1, N, K)) return e;
+  if (K % kTileCols != 0) return MATGPTQ_ESHAPE;
   if (!planes_host || !codes_host) return MATGPTQ_ENULL;
   switch (bitwidth) {
     case 2: master_slice_impl<2>(planes_host, N, K, codes_host); break;

@@ -31,11 +31,20 @@ void check_bits_group(int64_t bitwidth, int64_t group_size, int64_t n_in_feature
   }
 }
 
-void check_tiling(int64_t n_out_features, int64_t n_in_features) {
+// The reference needs n_in_features % 64 == 0 (utils.cpp:174-184).  Here: a multiple of 128, or
+// (where the group size divides it: 32 and -1) such a multiple plus 64; `whole_tiles`: the
+// master-resident planes take multiples of 128 only.
+void check_tiling(int64_t n_out_features, int64_t n_in_features, bool whole_tiles = false) {
   TORCH_CHECK(n_out_features > 0 && n_out_features % 16 == 0,
               "n_out_features must be a positive multiple of 16, got ", n_out_features);
-  TORCH_CHECK(n_in_features > 0 && n_in_features % 128 == 0,
-              "n_in_features must be a positive multiple of 128, got ", n_in_features);
+  if (whole_tiles) {
+    TORCH_CHECK(n_in_features > 0 && n_in_features % 128 == 0,
+                "n_in_features must be a positive multiple of 128, got ", n_in_features);
+  } else {
+    TORCH_CHECK(n_in_features > 0 && (n_in_features % 128 == 0 || (n_in_features % 128 == 64 && n_in_features >= 192)),
+                "n_in_features must be a positive multiple of 128, or at least 192 and a multiple of 128 plus 64, got ",
+                n_in_features);
+  }
 }
 
 void check_abi(int code, const char* what) {
@@ -229,7 +238,7 @@ Tensor pack_matgptq_master_resident(const Tensor& qweights) {
   TORCH_CHECK(qweights.is_contiguous(), "qweights must be contiguous");
   TORCH_CHECK(qweights.dim() == 2, "qweights must be 2D (n_out_features, n_in_features)");
   const int64_t n = qweights.size(0), k = qweights.size(1);
-  check_tiling(n, k);
+  check_tiling(n, k, true);
   const at::Device dev = target_device(qweights);
   c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
   const int64_t words = n * k / 4;
@@ -252,7 +261,7 @@ Tensor unpack_matgptq_master_resident(const Tensor& planes, int64_t n_out_featur
   TORCH_CHECK(planes.dtype() == torch::kUInt32 && planes.dim() == 1 && planes.is_contiguous(),
               "master planes must be a contiguous 1D uint32 tensor");
   check_bits_group(bitwidth, -1, n_in_features);
-  check_tiling(n_out_features, n_in_features);
+  check_tiling(n_out_features, n_in_features, true);
   TORCH_CHECK(planes.size(0) == n_out_features * n_in_features / 4, "master planes have the wrong size");
   Tensor out = torch::empty({n_out_features, n_in_features}, planes.options().dtype(torch::kUInt8));
   if (planes.is_cuda()) {

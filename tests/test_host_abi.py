@@ -87,6 +87,27 @@ def test_pack_from_master_slices_like_the_oracle(b):
     assert np.array_equal(_unpack(_pack(q, b, 1), 16, 128, b), o.slice_codes(q, b))
 
 
+@pytest.mark.parametrize("b", BITS)
+def test_pack_unpack_identity_with_a_tail_of_64_columns(b):
+    # K = 128 t + 64: tiles first, then the last 64 columns of every row as a bitstream; the size
+    # stays bitwidth * N * K / 32 words
+    rng = np.random.default_rng(20 + b)
+    for n, k in ((16, 192), (48, 128 * 3 + 64)):
+        c = rng.integers(0, 1 << b, (n, k), dtype=np.uint8)
+        packed = _pack(c, b)
+        assert packed.size == b * n * k // 32
+        assert np.array_equal(_unpack(packed, n, k, b), c)
+        q = rng.integers(0, 256, (n, k), dtype=np.uint8)
+        assert np.array_equal(_unpack(_pack(q, b, 1), n, k, b), o.slice_codes(q, b))
+    # the tail of a row is a plain little-endian bitstream: code j at bit j * b
+    c = np.zeros((16, 192), dtype=np.uint8)
+    c[5, 128 + 7] = (1 << b) - 1
+    words = _pack(c, b)[64 * b:].reshape(16, 2 * b)  # behind the one tile of 64 b words
+    bits = np.unpackbits(words[5].view(np.uint8), bitorder="little")
+    assert bits.sum() == b and np.all(bits[7 * b:8 * b] == 1)
+    assert not words[np.arange(16) != 5].any()
+
+
 def test_pack_ignores_bits_above_the_bitwidth():
     rng = np.random.default_rng(9)
     c = rng.integers(0, 256, (16, 128), dtype=np.uint8)
