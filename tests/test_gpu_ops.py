@@ -372,9 +372,11 @@ def test_torch_compile_fullgraph(mode):
     try:
         compiled = torch.compile(mod, fullgraph=True, mode=mode)
         got = [compiled(x).clone() for _ in range(4)]  # warm-up, capture and replays
+        print(f"torch.compile mode={mode}: inductor ran")
     except Exception as e:  # the inductor toolchain (a C++ compiler for its wrapper) may be absent
         if "fullgraph" in str(e).lower() or "graph break" in str(e).lower():
             raise
+        print(f"torch.compile mode={mode}: inductor unavailable ({type(e).__name__}), aot_eager instead")
         compiled = torch.compile(mod, fullgraph=True, backend="aot_eager")
         got = [compiled(x).clone() for _ in range(2)]
     torch.cuda.synchronize()

@@ -140,8 +140,15 @@ def test_error_codes():
     assert lib.matgptq_gemm(7, 128, 16, 128, 1, 1, 1, None, 1, 1, None, 1) == -1
     assert lib.matgptq_gemm(4, 48, 16, 128, 1, 1, 1, None, 1, 1, None, 1) == -2
     assert lib.matgptq_gemm(4, 128, 16, 128, 0, 1, 1, None, 1, 1, None, 1) == -8
-    for code in range(-8, 1):
-        assert lib.matgptq_strerror(code)
+    # 32-bit byte offsets inside the kernels: a packed tensor of 4 GiB or more is refused, and so is
+    # a dimension above 2^24 (no device work: the pointers are never touched)
+    assert lib.matgptq_gemm(8, 128, 65536, 65536, 1, 1, 1, None, 1, 1, None, 1) == -8
+    assert lib.matgptq_gemm(4, 128, 65536, 131072, 1, 1, 1, None, 1, 1, None, 1) == -8
+    assert lib.matgptq_gemm(2, 128, 16, 128, (1 << 24) + 1, 1, 1, None, 1, 1, None, 1) == -8
+    assert lib.matgptq_gemm(2, 128, 16, 1 << 25, 1, 1, 1, None, 1, 1, None, 1) == -8
+    assert lib.matgptq_gemm_master(2, 128, 65536, 65536, 1, 1, 1, None, 1, 1, None, 0, None, 1) == -8
+    for code in range(-10, 1):
+        assert lib.matgptq_strerror(code) != b"unknown error"
     with pytest.raises(_lib.MatGPTQError, match="bitwidth must be one of"):
         _lib.check(-1)
 
