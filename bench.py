@@ -246,6 +246,36 @@ def main() -> int:
     }
 
     extra = {}
+    # ------------------------------------------------------------- read floor
+    # What a kernel that only READ each layer's bytes takes on this GPU, measured the same way
+    # (graph replays, every launch on bytes no earlier launch of the replay touched): the bare-read
+    # probe of the library on the algorithmic bytes of each layer, and the four of a step in a row.
+    flat = torch.empty(int(RING_BYTES * 1.25) // 4, dtype=torch.int32, device=dev)
+    flat.random_(generator=g)
+    flat_bytes = flat.numel() * 4
+    cursor = [0]
+
+    def probe(nbytes):
+        nbytes = (nbytes + 4095) // 4096 * 4096
+        if cursor[0] + nbytes > flat_bytes:
+            cursor[0] = 0
+        _lib.check(L.matgptq_probe_read(flat.data_ptr() + cursor[0], nbytes, stream.cuda_stream))
+        cursor[0] += nbytes
+
+    layer_bytes = {name: algorithmic_bytes(n, k, 1, bits) for name, (n, k) in LLAMA3_8B.items()}
+    floor = {}
+    for name, nb in layer_bytes.items():
+        cnt = max(32, int(flat_bytes // nb))
+        t = timed_graph(lambda: [probe(nb) for _ in range(cnt)], reps=5) / cnt
+        floor[name] = {"us": round(t * 1e6, 2), "GBps": round(nb / t / 1e9, 1)}
+    t = timed_graph(lambda: [[probe(nb) for nb in layer_bytes.values()] for _ in range(args.steps)], reps=5) / args.steps
+    floor["step_of_four_reads_us"] = round(t * 1e6, 2)
+    floor["step_measured_over_floor"] = round(ms_per_step * 1e-3 / t, 3)
+    floor["dominant_kernel_over_its_read"] = round(t_dom * 1e6 / floor["gate_up"]["us"], 3)
+    extra["read_floor"] = floor
+    del flat
+    torch.cuda.empty_cache()
+
     cpu_baseline = None
     if not args.quick:
         # ------------------------------------------------- per layer, per bitwidth
@@ -419,6 +449,41 @@ def main() -> int:
             del wd
             torch.cuda.empty_cache()
         extra["speedup_over_dense_fp16"] = speed
+        # ---------------------------------------------------------- load time
+        # What process_weights_after_loading costs per layer (gate_up of Llama-3-8B, 117 M master
+        # codes already in HBM): slice + pack in one kernel (reads 1 byte per code, writes b/8),
+        # the master-resident planes (1 read, 1 written), the scale reorder; and the host packer
+        # (the reference's route: inference_lib/matgptq_cuda/csrc/bindings.cpp:63-83) on a 4096 x 4096
+        # layer with all host threads, without its two PCIe copies.
+        n, k = LLAMA3_8B["gate_up"]
+        master = torch.randint(0, 256, (n, k), dtype=torch.uint8, device=dev, generator=g)
+        load = {}
+        for b in (2, 4, 8):
+            out_words = torch.empty(L.matgptq_packed_words(b, n, k), dtype=torch.int32, device=dev)
+            t = timed_graph(lambda: _lib.check(L.matgptq_pack_device(master.data_ptr(), n, k, b, 1, out_words.data_ptr(),
+                                                                    torch.cuda.current_stream().cuda_stream)), reps=3)
+            moved = n * k * (1 + b / 8)
+            load[f"slice_pack_b{b}_gate_up"] = {"us": round(t * 1e6, 1), "GBps": round(moved / t / 1e9, 1),
+                                               "pct_hbm_peak": round(moved / t / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+            del out_words
+        planes = torch.empty(L.matgptq_master_words(n, k), dtype=torch.int32, device=dev)
+        t = timed_graph(lambda: _lib.check(L.matgptq_pack_master_device(master.data_ptr(), n, k, planes.data_ptr(),
+                                                                       torch.cuda.current_stream().cuda_stream)), reps=3)
+        load["master_planes_gate_up"] = {"us": round(t * 1e6, 1), "GBps": round(2 * n * k / t / 1e9, 1),
+                                         "pct_hbm_peak": round(2 * n * k / t / 1e9 / HBM_PEAK_GBPS * 100, 1)}
+        del planes, master
+        import numpy as np
+        hq = np.random.default_rng(0).integers(0, 256, (4096, 4096), dtype=np.uint8)
+        hout = np.zeros(L.matgptq_packed_words(4, 4096, 4096), dtype=np.uint32)
+        best = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            _lib.check(L.matgptq_pack_host(hq.ctypes.data, 4096, 4096, 4, 1, hout.ctypes.data))
+            best = min(best, time.perf_counter() - t0)
+        load["host_slice_pack_b4_4096x4096"] = {"ms": round(best * 1e3, 2), "Mcodes_per_s": round(4096 * 4096 / best / 1e6, 1),
+                                                "threads": os.cpu_count()}
+        extra["load_time"] = load
+        torch.cuda.empty_cache()
         # ---------------------------------------------------------- CPU baseline
         cpu_baseline = cpu_path_baseline(step_bytes)
 

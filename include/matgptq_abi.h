@@ -131,6 +131,12 @@ int matgptq_dequantize_device(int bitwidth, int group_size, int64_t N, int64_t K
                               const void *packed_dev, const void *scales_dev,
                               const void *zeros_dev, void *w_dev, void *stream);
 
+/* Measurement aid (no counterpart in the reference): streams `bytes` of device memory once through
+ * the load pattern of the batch-1 kernel (a wave requests four KiB-sized pieces at once, eight
+ * waves per workgroup) and does nothing with them.  bench.py times it on buffers of the size of a
+ * layer to state what a kernel that only read the weights would take on the same GPU. */
+int matgptq_probe_read(const void *buf_dev, size_t bytes, void *stream);
+
 /* ---- master-resident codes ------------------------------------------------------
  * The reference slices the 8-bit master codes once on the host, packs the slice and deletes
  * the master codes (inference_lib/vllm_matgptq.py:154-178,

@@ -24,6 +24,7 @@ EXPORTS = (
     "matgptq_master_words", "matgptq_pack_master_host", "matgptq_pack_master_device",
     "matgptq_unpack_master_host", "matgptq_unpack_master_device",
     "matgptq_gemm_master_workspace_bytes", "matgptq_gemm_master", "matgptq_gemm_master_static",
+    "matgptq_probe_read",
 )
 
 _lib = None
@@ -85,6 +86,8 @@ def load() -> ctypes.CDLL:
     L.matgptq_gemm_master.restype = ci
     L.matgptq_gemm_master_static.argtypes = [ci, ci, i64, i64, i64, vp, vp, vp, vp, vp, vp, u32]
     L.matgptq_gemm_master_static.restype = ci
+    L.matgptq_probe_read.argtypes = [vp, ctypes.c_size_t, vp]
+    L.matgptq_probe_read.restype = ci
     _lib = L
     return L
 

@@ -45,6 +45,7 @@ hipError_t launch_pack_master(const uint8_t*, int64_t, int64_t, uint32_t*, hipSt
 hipError_t launch_master_slice(const uint32_t*, int64_t, int64_t, int, bool, void*, hipStream_t);
 hipError_t launch_reorder(const uint16_t*, int64_t, int64_t, uint16_t*, hipStream_t);
 hipError_t launch_tail_gemm(int bits, bool bf16, const GemmArgs&, int group_size, hipStream_t);
+hipError_t launch_read_probe(const void*, size_t, hipStream_t);
 hipError_t launch_dequant(int, int, int64_t, int64_t, const uint32_t*, const uint16_t*,
                           const uint16_t*, uint16_t*, hipStream_t);
 
@@ -527,6 +528,13 @@ int matgptq_unpack_master_device(const uint32_t* planes_dev, int64_t N, int64_t 
   if (!planes_dev || !codes_dev) return MATGPTQ_ENULL;
   return launch_master_slice(planes_dev, N, K, bitwidth, false, codes_dev, static_cast<hipStream_t>(stream)) ==
                  hipSuccess ? MATGPTQ_OK : MATGPTQ_ELAUNCH;
+}
+
+int matgptq_probe_read(const void* buf_dev, size_t bytes, void* stream) {
+  if (!buf_dev) return MATGPTQ_ENULL;
+  if (bytes == 0 || bytes % 16 != 0) return MATGPTQ_ESIZE;
+  return launch_read_probe(buf_dev, bytes, static_cast<hipStream_t>(stream)) == hipSuccess ? MATGPTQ_OK
+                                                                                          : MATGPTQ_ELAUNCH;
 }
 
 int matgptq_describe_plan(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
