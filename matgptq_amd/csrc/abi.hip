@@ -438,8 +438,7 @@ static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t 
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zp, flags, &p)) return e;
-  // (the gemv kernel reads the planes directly at group size 128)
-  *direct = p.gemv && group_size == 128 && (p.shape == 1 || p.shape == 2);
+  *direct = p.gemv && (p.shape == 1 || p.shape == 2);
   return MATGPTQ_OK;
 }
 

@@ -347,7 +347,7 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 // Entry of this translation unit.  shape: index into the (T, R) table above; W: waves per
 // workgroup (1..16); lds_pad: dynamic LDS to ask for when it exceeds what the kernel needs
 // (limits how many workgroups share a CU); master: `a.packed` holds master-resident bit planes
-// (shapes 1 and 2, group size 128 only); group sizes 32 and -1: shapes 1 and 2.  M <= 4 only.
+// (shapes 1 and 2); group sizes 32 and -1: shapes 1 and 2.  M <= 4 only.
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 #if MATGPTQ_BF16
@@ -357,8 +357,12 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 #endif
 hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int shape, int W, size_t lds_pad, bool master,
                                hipStream_t stream) {
-  if (group_size == 32) return master ? hipErrorInvalidValue : launch_storage<32, false>(a, shape, W, lds_pad, stream);
-  if (group_size == -1) return master ? hipErrorInvalidValue : launch_storage<-1, false>(a, shape, W, lds_pad, stream);
+  if (group_size == 32)
+    return master ? launch_storage<32, true>(a, shape, W, lds_pad, stream)
+                  : launch_storage<32, false>(a, shape, W, lds_pad, stream);
+  if (group_size == -1)
+    return master ? launch_storage<-1, true>(a, shape, W, lds_pad, stream)
+                  : launch_storage<-1, false>(a, shape, W, lds_pad, stream);
   return master ? launch_storage<128, true>(a, shape, W, lds_pad, stream)
                 : launch_storage<128, false>(a, shape, W, lds_pad, stream);
 }

@@ -54,24 +54,25 @@ def test_device_pack_equals_host_pack_and_slices_bit_exactly(golden):
         assert np.array_equal(back.cpu().numpy(), o.slice_codes(q, b)), b
 
 
+@pytest.mark.parametrize("g", (128, 32, -1))
 @pytest.mark.parametrize("zp", (False, True))
-def test_every_bitwidth_from_one_buffer(zp):
+def test_every_bitwidth_from_one_buffer(zp, g):
     # 5 row blocks, 13 K tiles: ragged for two row blocks per workgroup and for the rounds
     n, k = 80, 128 * 13
-    q, s, z = o.make_layer(n, k, 128, seed=11, symmetric=not zp)
+    q, s, z = o.make_layer(n, k, g, seed=11, symmetric=not zp)
     planes = planes_device(q)
-    sc = G.reorder_device(s, n, k, 128)
-    zr = G.reorder_device(z, n, k, 128) if zp else None
+    sc = G.reorder_device(s, n, k, g)
+    zr = G.reorder_device(z, n, k, g) if zp else None
     for b in BITS:
-        w = o.dequantize(q, s, z, b, 128)
+        w = o.dequantize(q, s, z, b, g)
         for m in (1, 2, 3, 4):
             x = o.make_activations(m, k, seed=m + b)
-            y, need = gemm_master(b, 128, n, k, G.to_dev(x), planes, sc, zr)
+            y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zr)
             assert need == 0  # the kernel reads the planes itself
             G.assert_close_to_oracle(y, x, w, f"master planes b={b} zp={zp} M={m}")
             G.assert_regression_bound(y, x, w, f"master planes b={b} zp={zp} M={m}")
             # the same product on the pre-sliced tensor: same codes, same arithmetic
-            y2 = G.gemm(b, 128, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zr).cpu().numpy()
+            y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zr).cpu().numpy()
             assert np.max(np.abs(y.astype(np.float64) - y2)) <= 2.0 ** -9 * np.max(np.abs(y2))
 
 
@@ -90,7 +91,7 @@ def test_exact_in_the_reference_test_regime():
             assert np.array_equal(y.view(np.uint16), o.linear_f64(x, w).astype(np.float16).view(np.uint16)), (b, m)
 
 
-@pytest.mark.parametrize("b,g,m", [(4, 128, 8), (3, 128, 16), (4, 128, 64), (6, 128, 300), (2, 32, 1), (8, -1, 3), (4, 32, 40)])
+@pytest.mark.parametrize("b,g,m", [(4, 128, 8), (3, 128, 16), (4, 128, 64), (6, 128, 300), (2, 32, 5), (8, -1, 13), (4, 32, 40)])
 def test_shapes_outside_the_gemv_kernel_go_through_the_workspace(b, g, m):
     n, k = 304, 1024
     q, s, z = o.make_layer(n, k, g, seed=b + m)
