@@ -218,7 +218,7 @@ def main() -> int:
         stream.synchronize()
     torch.cuda.synchronize()
     t_wall0 = time.perf_counter()
-    elapsed = timed_graph(lambda: [step(i) for i in range(args.steps)], reps=7)  # median of 7 replays
+    elapsed = timed_graph(lambda: [step(i) for i in range(args.steps)], reps=21)  # median of 21 replays
     torch.cuda.synchronize()
     t_wall = time.perf_counter() - t_wall0
     ms_per_step = elapsed / args.steps * 1e3
@@ -230,7 +230,7 @@ def main() -> int:
     t_dom = timed_graph(lambda: [launch(bits, n, k, x_ring["gate_up"][i % copies], rings["gate_up"][i % copies],
                                         aux_ring["gate_up"][i % copies][0], aux_ring["gate_up"][i % copies][1],
                                         ys["gate_up"])
-                                 for i in range(launches)], reps=7) / launches
+                                 for i in range(launches)], reps=21) / launches
     dom_bytes = algorithmic_bytes(n, k, 1, bits)
     roofline = {
         "kernel": _lib.describe_plan(bits, GROUP, n, k, 1, True),
