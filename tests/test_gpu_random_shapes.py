@@ -1,0 +1,40 @@
+"""Seeded random problems through the planner's default choice: whatever kernel it picks for a
+shape, the result must match the oracle.  Row counts that leave ragged row blocks for every
+workgroup shape, K from one tile to long walks (with and without the 64-column tail), every
+batch regime, bitwidth, group size and zero-point form."""
+import numpy as np
+import pytest
+
+from matgptq_amd import _lib
+from oracle import matgptq_oracle as o
+from tests import _gpu_util as G
+
+pytestmark = pytest.mark.gpu
+BITS = (2, 3, 4, 6, 8)
+
+
+def _cases(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        b = int(rng.choice(BITS))
+        g = int(rng.choice((128, 128, 32, -1)))
+        n = 16 * int(rng.integers(1, 41))
+        tiles = int(rng.choice((1, 2, 3, 5, 8, 13, 16, 27, 32)))
+        k = 128 * tiles + (64 if g != 128 and tiles >= 1 and rng.random() < 0.3 else 0)
+        m = int(rng.choice((1, 2, 3, 4, 5, 7, 8, 12, 16, 17, 31, 33, 64, 100, 129, 257)))
+        zp = bool(rng.integers(0, 2))
+        out.append((b, g, n, k, m, zp))
+    return out
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_problems_through_the_default_plan(seed):
+    for b, g, n, k, m, zp in _cases(seed, 25):
+        lay = G.Layer(n, k, b, g, seed=seed * 1000 + n + k + m, zero_points=zp)
+        x = o.make_activations(m, k, seed=seed + m, outlier_frac=0.01)
+        plan = _lib.describe_plan(b, g, n, k, m, zp)
+        y = lay.run(x)
+        what = f"b={b} g={g} N={n} K={k} M={m} zp={zp} [{plan}]"
+        G.assert_close_to_oracle(y, x, lay.w, what)
+        G.assert_regression_bound(y, x, lay.w, what)
