@@ -54,8 +54,9 @@ namespace {
 constexpr int kDecodeMaxM = 16;
 constexpr int kGemvMaxM = 4;
 // (tiles per wave and round, row blocks per workgroup) of the gemv kernel's instantiations
-constexpr int kNumGemvShapes = 6;
-constexpr int kGemvShapes[kNumGemvShapes][2] = {{8, 1}, {4, 1}, {4, 2}, {2, 2}, {2, 4}, {2, 1}};
+// (group sizes 32 and -1 and the master-resident planes: entries 1 and 2 only)
+constexpr int kNumGemvShapes = 7;
+constexpr int kGemvShapes[kNumGemvShapes][2] = {{8, 1}, {4, 1}, {4, 2}, {2, 2}, {2, 4}, {2, 1}, {4, 4}};
 constexpr size_t kLdsBudget = 64 * 1024;  // dynamic LDS a decode workgroup may ask for
 
 struct Plan {
@@ -210,6 +211,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   // Group sizes 32 and -1 run the two shapes named here (a scale per octet, or per row).
   if (M <= kGemvMaxM && flavour == 0 && (variant == 0 || variant >= 100)) {
     int shape = ((M >= 2 && row_blocks >= 320) || (bits == 2 && group_size == 128 && row_blocks >= 1024)) ? 2 : 1;
+    // several batch rows, 2 or 3 bits, many row blocks: four row blocks per workgroup halve the
+    // activations re-read from L2 once more and their codes still fit the registers of eight waves
+    // per SIMD (28672 x 4096 at M = 4: 3 bits 11.8 against 13.1 us, 2 bits 9.35 against 10.0;
+    // 4 bits 14.9 against 13.5: its 64 registers of codes leave four waves per SIMD)
+    if (M >= 2 && bits <= 3 && group_size == 128 && row_blocks >= 1024) shape = 6;
     if (variant >= 100) {
       shape = variant - 100;
       if (shape >= kNumGemvShapes) return MATGPTQ_EVARIANT;

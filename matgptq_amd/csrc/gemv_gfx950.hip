@@ -327,6 +327,7 @@ hipError_t launch_shape(const GemmArgs& a, int shape, int W, size_t lds_pad, hip
       case 2: return launch_one<ZP, 128, 4, 2, MB, 4, false>(a, W, lds_pad, s);
       case 3: return launch_one<ZP, 128, 2, 2, MB, 4, false>(a, W, lds_pad, s);
       case 4: return launch_one<ZP, 128, 2, 4, MB, 4, false>(a, W, lds_pad, s);
+      case 6: return launch_one<ZP, 128, 4, 4, MB, 4, false>(a, W, lds_pad, s);
       default: return launch_one<ZP, 128, 2, 1, MB, 4, false>(a, W, lds_pad, s);
     }
   }

@@ -13,13 +13,14 @@ pytestmark = pytest.mark.gpu
 LLAMA8B = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "down": (4096, 14336)}
 LLAMA70B = {"qkv": (10240, 8192), "o": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
 
-# kernel the planner takes per layer and batch size (4 and 3 bits take the same)
+# kernel the planner takes per layer and batch size (4 and 3 bits take the same, except that 3 bits
+# take four row blocks per workgroup on the layer with many rows: `{r}`)
 SMALL_BATCH_PLANS = {
     "qkv": {2: "gemv b{b} g128 zp1 T4 R2 W8 pad0", 4: "gemv b{b} g128 zp1 T4 R2 W8 pad0",
             8: "midbatch b{b} g128 zp1 R2 mb1", 16: "midbatch b{b} g128 zp1 R2 mb1"},
     "o": {2: "gemv b{b} g128 zp1 T4 R1 W8 pad0", 4: "gemv b{b} g128 zp1 T4 R1 W8 pad0",
           8: "midbatch b{b} g128 zp1 R1 mb1", 16: "midbatch b{b} g128 zp1 R1 mb1"},
-    "gate_up": {2: "gemv b{b} g128 zp1 T4 R2 W8 pad0", 4: "gemv b{b} g128 zp1 T4 R2 W8 pad0",
+    "gate_up": {2: "gemv b{b} g128 zp1 T4 R{r} W8 pad0", 4: "gemv b{b} g128 zp1 T4 R{r} W8 pad0",
                 8: "midbatch b{b} g128 zp1 R4 mb1", 16: "midbatch b{b} g128 zp1 R4 mb1"},
     "down": {2: "gemv b{b} g128 zp1 T4 R1 W16 pad0", 4: "gemv b{b} g128 zp1 T4 R1 W16 pad0",
              8: "midbatch b{b} g128 zp1 R1 mb1", 16: "midbatch b{b} g128 zp1 R1 mb1"},
@@ -33,7 +34,7 @@ def test_config2_small_batch_full_size(name, b):
     n, k = LLAMA8B[name]
     lay = G.Layer(n, k, b, 128, seed=100 + b)
     for m in (2, 4, 8, 16):
-        assert _lib.describe_plan(b, 128, n, k, m, True) == SMALL_BATCH_PLANS[name][m].format(b=b)
+        assert _lib.describe_plan(b, 128, n, k, m, True) == SMALL_BATCH_PLANS[name][m].format(b=b, r=4 if b <= 3 else 2)
         x = o.make_activations(m, k, seed=m, outlier_frac=0.01, outlier_gain=20.0)
         y = lay.run(x)
         G.assert_close_to_oracle(y, x, lay.w, f"{name} b={b} M={m}")

@@ -14,7 +14,7 @@ from tests import _gpu_util as G
 
 pytestmark = pytest.mark.gpu
 BITS = (2, 3, 4, 6, 8)
-SHAPES = range(6)  # (T, R) entries of the kernel: (8,1) (4,1) (4,2) (2,2) (2,4) (2,1)
+SHAPES = range(7)  # (T, R) entries of the kernel: (8,1) (4,1) (4,2) (2,2) (2,4) (2,1) (4,4)
 
 
 def gemv_flags(shape, waves=0, base=1):
@@ -100,7 +100,7 @@ def test_gemv_is_not_taken_outside_its_domain():
     with pytest.raises(_lib.MatGPTQError, match="variant"):
         G.Layer(32, 256, 4, 128, seed=1).run(o.make_activations(5, 256, seed=1), flags=gemv_flags(0))
     with pytest.raises(_lib.MatGPTQError, match="variant"):
-        G.Layer(32, 256, 4, 128, seed=1).run(o.make_activations(1, 256, seed=1), flags=gemv_flags(6))
+        G.Layer(32, 256, 4, 128, seed=1).run(o.make_activations(1, 256, seed=1), flags=gemv_flags(7))
 
 
 @pytest.mark.parametrize("b", (2, 4, 8))

@@ -163,11 +163,13 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(4, 32, 4096, 4096, 1) == "gemv b4 g32 zp0 T4 R1 W8 pad0"
     assert _lib.describe_plan(4, -1, 4096, 4096, 4) == "gemv b4 g-1 zp0 T4 R1 W8 pad0"
     assert _lib.describe_plan(2, 128, 28672, 4096, 1, True) == "gemv b2 g128 zp1 T4 R2 W8 pad0"
+    assert _lib.describe_plan(3, 128, 28672, 4096, 4, True) == "gemv b3 g128 zp1 T4 R4 W8 pad0"
+    assert _lib.describe_plan(3, 128, 6144, 4096, 4, True) == "gemv b3 g128 zp1 T4 R2 W8 pad0"
     assert _lib.describe_plan(4, 32, 4096, 4096, 5).startswith(("decode", "midbatch"))
     assert _lib.describe_plan(4, 128, 28672, 4096, 5, True).startswith("decode")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048).startswith("prefill")
     with pytest.raises(RuntimeError):
-        _lib.describe_plan(4, 128, 4096, 4096, 1, True, 1 | (106 << 8))   # no such gemv entry
+        _lib.describe_plan(4, 128, 4096, 4096, 1, True, 1 | (107 << 8))   # no such gemv entry
     with pytest.raises(RuntimeError):
         _lib.describe_plan(4, 128, 4096, 4096, 1, True, 1 | (100 << 8) | (17 << 18))  # more than 16 waves
     with pytest.raises(RuntimeError):
