@@ -127,3 +127,30 @@ def test_torch_ops_and_module_with_tail():
         x = o.make_activations(m, k, seed=m)
         y = lin(torch.from_numpy(x).to(G.DEV)).cpu().numpy()
         G.assert_close_to_oracle(y, x, w, f"module M={m}")
+
+
+def test_gemm_with_tail_in_a_graph():
+    # two launches (tiles, then the tail): both capturable; replays, with eager work of the same
+    # operator between them, are checked against the eager result
+    n, k, b, g = 128, 128 * 6 + 64, 4, 32
+    lay = G.Layer(n, k, b, g, seed=5)
+    for m in (1, 40):
+        x = G.to_dev(o.make_activations(m, k, seed=m))
+        eager = G.gemm(b, g, n, k, x, lay.packed, lay.scales, lay.zeros).clone()
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream()
+        y = torch.empty((m, n), dtype=torch.float16, device=G.DEV)
+        with torch.cuda.stream(stream):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                _lib.check(G.lib().matgptq_gemm(b, g, n, k, m, lay.packed.data_ptr(), lay.scales.data_ptr(),
+                                                lay.zeros.data_ptr(), x.data_ptr(), y.data_ptr(),
+                                                stream.cuda_stream, 1))
+            for _ in range(3):
+                y.fill_(float("nan"))
+                graph.replay()
+                stream.synchronize()
+                assert torch.equal(y, eager), m
+                other = G.gemm(b, g, n, k, x, lay.packed, lay.scales, lay.zeros)
+                torch.cuda.synchronize()
+                assert torch.equal(other, eager)
