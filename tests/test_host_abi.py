@@ -219,3 +219,16 @@ def test_planner_keeps_six_bit_codes_off_the_largest_ring_tile():
     assert _lib.describe_plan(8, 128, 10240, 8192, 2048, True).endswith("cfg8")
     assert _lib.describe_plan(8, 128, 8192, 8192, 2048, False).endswith("cfg0")
     assert _lib.describe_plan(3, 128, 8192, 8192, 2048, True).endswith("cfg0")
+
+
+def test_header_is_plain_c(tmp_path):
+    # the boundary is a C ABI: the header has to compile as C99 with nothing but the standard headers
+    import shutil
+    import subprocess
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "t.c"
+    src.write_text('#include "matgptq_abi.h"\nint main(void) { return matgptq_abi_version() == 0; }\n')
+    subprocess.run([cc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    "-c", str(src), "-o", str(tmp_path / "t.o")], check=True)
