@@ -38,3 +38,38 @@ def test_random_problems_through_the_default_plan(seed):
         what = f"b={b} g={g} N={n} K={k} M={m} zp={zp} [{plan}]"
         G.assert_close_to_oracle(y, x, lay.w, what)
         G.assert_regression_bound(y, x, lay.w, what)
+
+
+def _bf16_dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(G.DEV)
+
+
+@pytest.mark.parametrize("seed", (10, 11))
+def test_random_problems_bf16_storage(seed):
+    import torch
+    L = G.lib()
+    for b, g, n, k, m, zp in _cases(seed, 20):
+        q, s16, z16 = o.make_layer(n, k, g, seed=seed * 1000 + n + k + m, symmetric=not zp)
+        s = o.round_to_bf16(s16.astype(np.float32))
+        z = z16.astype(np.float32)
+        x = o.round_to_bf16(o.make_activations(m, k, seed=seed + m, outlier_frac=0.01).astype(np.float32))
+        pk = G.pack_device(q, b, True)
+
+        def reorder(a):
+            src = _bf16_dev(a)
+            out = torch.empty_like(src)
+            _lib.check(L.matgptq_reorder_scales_device(src.data_ptr(), n, k, g, out.data_ptr(), G.stream()))
+            return out
+
+        sr = reorder(s)
+        zr = reorder(z) if zp else None
+        y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=G.DEV)
+        _lib.check(L.matgptq_gemm(b, g, n, k, m, pk.data_ptr(), sr.data_ptr(), zr.data_ptr() if zp else None,
+                                  _bf16_dev(x).data_ptr(), y.data_ptr(), G.stream(), 3))
+        torch.cuda.synchronize()
+        yv = y.float().cpu().numpy()
+        ref = o.linear_f64(x, o.dequantize_bf16(q, s, z, b, g))
+        what = f"bf16 b={b} g={g} N={n} K={k} M={m} zp={zp} [{_lib.describe_plan(b, g, n, k, m, zp, 3)}]"
+        assert np.all(np.isfinite(yv)), what
+        assert np.max(np.abs(yv - ref)) <= G.REL_TOL * np.max(np.abs(ref)), what
