@@ -148,12 +148,18 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // instructions per pair of weights instead of two): the wider tiles spill or stall on that
       // work, the 128 x 128 tile does not, and up to 4 bits neither does the 128 x 192 tile
       // (Llama-3-70B gate_up, M = 2048, 4 bits: 1590 against 1768 us; the 128 x 256 tile takes 2241).
+      // Group size 32 with zero points keeps four scales and four zeros per tile and row block in
+      // two register sets: the 128 x 256 tile spills (8192 x 8192, M = 2048: 489 us at 4 bits, 3023 us
+      // at 8 bits, against 290 and 307 us on the 128 x 128 tile); the 128 x 192 tile fits up to 4 bits
+      // and at 8 (57344 x 8192, 4 bits: 1728 against 1902 us).
       const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
-      if (bits == 6 || bf16) {
+      const bool g32zp = group_size == 32 && zp;
+      if (bits == 6 || bf16 || g32zp) {
         const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
         const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
         const double t_128 = (double)((wgs_128 + 511) / 512);
-        p->cfg = t_192 < t_128 && (bits <= 4 || !bf16) ? 9 : 3;
+        const bool fits_192 = !(bf16 && (bits > 4 || group_size == 32)) && !(bits == 6 && g32zp);
+        p->cfg = t_192 < t_128 && fits_192 ? 9 : 3;
       }
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X

@@ -159,3 +159,24 @@ def test_prefill_zero_point_form_deviation_per_weight():
     ulp_w = np.maximum(np.abs(w), 2.0 ** -14) * 2.0 ** -10
     ulp_term = 128.0 * s * 2.0 ** -11
     assert np.all(np.abs(w_eff - w) <= ulp_w + ulp_term + 1e-12)
+
+
+@pytest.mark.parametrize("b,g,plan", [(4, 32, "prefill b4 g32 zp1 cfg3"), (8, 32, "prefill b8 g32 zp1 cfg3"),
+                                      (4, -1, "prefill b4 g-1 zp1 cfg0")])
+def test_prefill_other_group_sizes_full_size(b, g, plan):
+    # the Llama-3-70B o layer at M = 2048 with a scale and a zero per 32 columns (kept off the tile
+    # whose registers they do not fit) and per row
+    n, k = LLAMA70B["o"]
+    m = 2048
+    assert _lib.describe_plan(b, g, n, k, m, True) == plan
+    q, s, z = o.make_layer(n, k, g, seed=17)
+    x = o.make_activations(m, k, seed=12)
+    packed = G.pack_device(q, b, True)
+    sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
+    y = G.gemm(b, g, n, k, G.to_dev(x), packed, sc, zr)
+    torch.cuda.synchronize()
+    rows = np.array([t * 128 + (37 * t + 5) % 128 for t in range(16)])
+    yr = y[torch.from_numpy(rows).to(G.DEV)].cpu().numpy()
+    assert bool(torch.isfinite(y.float()).all())
+    ref, bound = G.oracle_product_in_chunks(q, s, z, b, g, x[rows])
+    G.assert_close_to_reference(yr, ref, bound, f"70B o prefill b={b} g={g}")

@@ -196,6 +196,16 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
 
 
+def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
+    # four scales and four zeros per tile and row block in two register sets spill there
+    assert _lib.describe_plan(4, 32, 8192, 8192, 2048, True).endswith("cfg3")
+    assert _lib.describe_plan(8, 32, 8192, 8192, 2048, True).endswith("cfg3")
+    assert _lib.describe_plan(4, 32, 57344, 8192, 2048, True).endswith("cfg9")
+    assert _lib.describe_plan(6, 32, 57344, 8192, 2048, True).endswith("cfg3")
+    assert _lib.describe_plan(4, 32, 8192, 8192, 2048, False).endswith("cfg0")   # scales alone fit
+    assert _lib.describe_plan(4, -1, 8192, 8192, 2048, True).endswith("cfg0")
+
+
 def test_planner_gives_bf16_storage_the_narrower_ring_tiles():
     # bf16 weights are formed in fp32 (twice the vector work per weight): the 128 x 256 tile stalls
     # on it; 128 x 192 up to 4 bits where its rounds pay, else 128 x 128.  Every tile can be forced.
