@@ -194,13 +194,14 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     }
   } else if (flavour == 0 &&
              (row_blocks < 1024 ? (M >= 8 || (M >= 4 && k_tiles >= 64) || (M >= 2 && k_tiles >= 112))
-                                : (M >= 8 && r_max == 4))) {
+                                : (M >= 8 && (r_max == 4 || (group_size == 32 && bits <= 4))))) {
     // Small batches: every decode workgroup stages the whole batch of activations (scaled
     // copies, written by the vector ALU), which grows with M and K, while the mid-batch kernel
     // copies them into LDS asynchronously.  Measured on MI355X (Llama-3-8B and 70B layers, 3 and
     // 4 bits): the latter wins from eight batch rows on, and earlier on layers with few rows
     // and a long K; on layers with many rows only where it may take four row blocks per
-    // workgroup.
+    // workgroup, or, at group size 32 (two row blocks at most), up to 4 bits (28672 x 4096 at M = 8,
+    // group 32: 4 bits 20.9 against 28.2 us, 2 bits 18.6 against 26.4; 8 bits tie at 29).
     p->decode = false;
     p->skinny = true;
     p->mb = 1;
