@@ -192,16 +192,16 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         }
       }
     }
-  } else if (flavour == 0 &&
-             (row_blocks < 1024 ? (M >= 8 || (M >= 4 && k_tiles >= 64) || (M >= 2 && k_tiles >= 112))
-                                : (M >= 8 && (r_max == 4 || (group_size == 32 && bits <= 4))))) {
-    // Small batches: every decode workgroup stages the whole batch of activations (scaled
-    // copies, written by the vector ALU), which grows with M and K, while the mid-batch kernel
-    // copies them into LDS asynchronously.  Measured on MI355X (Llama-3-8B and 70B layers, 3 and
-    // 4 bits): the latter wins from eight batch rows on, and earlier on layers with few rows
-    // and a long K; on layers with many rows only where it may take four row blocks per
-    // workgroup, or, at group size 32 (two row blocks at most), up to 4 bits (28672 x 4096 at M = 8,
-    // group 32: 4 bits 20.9 against 28.2 us, 2 bits 18.6 against 26.4; 8 bits tie at 29).
+  } else if (flavour == 0 && M > kGemvMaxM &&
+             (row_blocks < 1024 || r_max == 4 || (group_size == 32 && bits <= 4))) {
+    // Five to sixteen batch rows (one to four go to the gemv kernel below): every decode
+    // workgroup stages the whole batch of activations (scaled copies, written by the vector
+    // ALU), which grows with M and K, while the mid-batch kernel copies them into LDS
+    // asynchronously.  Measured on MI355X (Llama-3-8B layers, 2, 4 and 8 bits, M = 5 .. 16, weights
+    // cold): the mid-batch kernel wins everywhere (M = 7, 4 bits: 4096 x 4096 5.4 against 7.3 us,
+    // 6144 x 4096 6.1 against 8.5, 28672 x 4096 15.8 against 20.4) except on layers with many
+    // rows where it may take two row blocks only: 8 bits (28672 x 4096: 24.8 against 23.7 us), and
+    // group size 32 above 4 bits (at 4 bits, M = 8: 20.9 against 28.2 us; 8 bits tie at 29).
     p->decode = false;
     p->skinny = true;
     p->mb = 1;
