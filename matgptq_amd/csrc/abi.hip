@@ -177,6 +177,15 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       const double t_128 = 1.33 * kt * (1.0 + 0.5 * second) * (wgs_128 > 512 ? (double)wgs_128 / 512.0 : 1.0);
       const double t_32 = 0.95 * kt * (wgs_32 > 512 ? (double)wgs_32 / 512.0 : 1.0);
       p->cfg = t_128 < t_32 ? 3 : 4;
+      // Where the 128 x 128 ring tiles would sit one per CU (it is built for two, whose waves cover
+      // each other's waits), the staged 64 x 256 tile - twice the row blocks per dequantised
+      // activation block, as many workgroups - is faster while its own workgroups fit one round
+      // (M = 512: 8192 x 8192 92 against 103 us, 8192 x 28672 297 against 370; 28672 x 4096 at M = 128: 48
+      // against 55).  fp16 storage, group sizes 128 and -1 (its registers hold no more).
+      const int64_t wgs_64 = ((N + 255) / 256) * ((M + 63) / 64);
+      if (p->cfg == 3 && wgs_128 <= 256 && wgs_64 <= 256 && wgs_64 >= 128 && group_size != 32 &&
+          !(flags & MATGPTQ_FLAG_BF16))
+        p->cfg = 2;
       double best = t_128 < t_32 ? t_128 : t_32;
       for (int mb = 2; mb <= (M > 32 ? 4 : 2); mb <<= 1) {
         const int64_t m_tiles = (M + 16 * mb - 1) / (16 * mb);

@@ -203,6 +203,15 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
 
 
+def test_planner_takes_the_staged_tile_where_ring_tiles_would_sit_one_per_cu():
+    assert _lib.describe_plan(4, 128, 8192, 8192, 512, True).endswith("cfg2")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).endswith("cfg2")
+    assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True).endswith("cfg3")    # two ring tiles per CU
+    assert _lib.describe_plan(4, 128, 10240, 8192, 512, True).endswith("cfg3")
+    assert _lib.describe_plan(4, 32, 8192, 8192, 512, True).endswith("cfg3")      # group 32: registers
+    assert _lib.describe_plan(4, 128, 8192, 8192, 512, True, 3).endswith("cfg3")  # bf16 storage
+
+
 def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
     # four scales and four zeros per tile and row block in two register sets spill there
     assert _lib.describe_plan(4, 32, 8192, 8192, 2048, True).endswith("cfg3")
