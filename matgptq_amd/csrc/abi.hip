@@ -146,7 +146,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // tiles of 192, it only ties).  Rounds times tile width decide.
       // bf16 storage dequantises through fp32 for the bf16 matrix instruction (four vector
       // instructions per pair of weights instead of two): the wider tiles spill or stall on that
-      // work, the 128 x 128 tile does not, and up to 4 bits neither does the 128 x 192 tile
+      // work, the 128 x 128 tile does not, and except at 6 bits neither does the 128 x 192 tile
       // (Llama-3-70B gate_up, M = 2048, 4 bits: 1590 against 1768 us; the 128 x 256 tile takes 2241).
       // Group size 32 with zero points keeps four scales and four zeros per tile and row block in
       // two register sets: the 128 x 256 tile spills (8192 x 8192, M = 2048: 489 us at 4 bits, 3023 us
@@ -158,7 +158,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
         const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
         const double t_128 = (double)((wgs_128 + 511) / 512);
-        const bool fits_192 = !(bf16 && (bits > 4 || group_size == 32)) && !(bits == 6 && g32zp);
+        const bool fits_192 = !(bf16 && (bits == 6 || group_size == 32)) && !(bits == 6 && g32zp);
         p->cfg = t_192 < t_128 && fits_192 ? 9 : 3;
       }
     } else {

@@ -224,11 +224,12 @@ def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
 
 def test_planner_gives_bf16_storage_the_narrower_ring_tiles():
     # bf16 weights are formed in fp32 (twice the vector work per weight): the 128 x 256 tile stalls
-    # on it; 128 x 192 up to 4 bits where its rounds pay, else 128 x 128.  Every tile can be forced.
+    # on it; 128 x 192 where its rounds pay (not at 6 bits: registers), else 128 x 128.  Every tile can be forced.
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3).endswith("cfg9")
     assert _lib.describe_plan(4, 128, 57344, 8192, 2048, False, 3).endswith("cfg9")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 3).endswith("cfg3")
-    assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True, 3).endswith("cfg3")
+    assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True, 3).endswith("cfg9")
+    assert _lib.describe_plan(6, 128, 57344, 8192, 2048, True, 3).endswith("cfg3")
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8)).endswith("cfg8")
 
 
