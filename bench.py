@@ -298,6 +298,32 @@ def main() -> int:
                     }
                 del ring
         extra["gemv_M1"] = table
+        # ------------- the same kernel on the Llama-3-70B layers (M = 1, 4 bits, scale + zero): larger
+        # layers amortise the launch and the first-byte latency that bound the 8-60 MB layers above
+        t70 = {}
+        step70_us, step70_bytes = 0.0, 0
+        for name, (n, k) in LLAMA3_70B.items():
+            wbytes = n * k * bits // 8
+            cp = max(2, int(RING_BYTES // wbytes) + 1)
+            ring = make_ring(n, k, bits, cp)
+            auxs = [make_aux(n, k) for _ in range(cp)]
+            x70 = torch.randn(1, k, device=dev, generator=g).to(torch.float16)
+            y70 = torch.empty(1, n, dtype=torch.float16, device=dev)
+            reps = max(cp, 16)
+            t = timed_graph(lambda: [launch(bits, n, k, x70, ring[i % cp], auxs[i % cp][0], auxs[i % cp][1], y70)
+                                     for i in range(reps)]) / reps
+            ab = algorithmic_bytes(n, k, 1, bits)
+            t70[name] = {"us": round(t * 1e6, 2), "weight_GBps": round(wbytes / t / 1e9, 1),
+                         "pct_hbm_peak": round(wbytes / t / 1e9 / HBM_PEAK_GBPS * 100, 1),
+                         "algorithmic_pct_hbm_peak": round(ab / t / 1e9 / HBM_PEAK_GBPS * 100, 1),
+                         "kernel": _lib.describe_plan(bits, GROUP, n, k, 1, True)}
+            step70_us += t * 1e6
+            step70_bytes += wbytes
+            del ring, auxs
+            torch.cuda.empty_cache()
+        t70["step_sum_of_layers"] = {"us": round(step70_us, 2), "weight_GBps": round(step70_bytes / step70_us / 1e3, 1),
+                                     "pct_hbm_peak": round(step70_bytes / step70_us / 1e3 / HBM_PEAK_GBPS * 100, 1)}
+        extra["gemv_M1_llama3_70b"] = t70
         # ----------------- master-resident planes: one buffer, bitwidth chosen per call (M = 1)
         # moved bytes per weight: (b + 1) / 8 for 2, 3 and 4 bits (the top b bits and the round bit),
         # 1 for 6 and 8 bits; both rates are stated, on the sliced bytes and on the bytes moved
