@@ -227,8 +227,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   // Group sizes 32 and -1 run the two shapes named here (a scale per octet, or per row).
   if (M <= kGemvMaxM && flavour == 0 && (variant == 0 || variant >= 100)) {
     int shape = ((M >= 2 && row_blocks >= 320) || (bits == 2 && group_size == 128 && row_blocks >= 1024)) ? 2 : 1;
-    // several batch rows, 2 or 3 bits, many row blocks: four row blocks per workgroup halve the
-    // activations re-read from L2 once more and their codes still fit the registers of eight waves
+    // several batch rows, 2 or 3 bits, many row blocks: four row blocks per workgroup share one
+    // staging of the activations and their codes still fit the registers of eight waves
     // per SIMD (28672 x 4096 at M = 4: 3 bits 11.8 against 13.1 us, 2 bits 9.35 against 10.0;
     // 4 bits 14.9 against 13.5: its 64 registers of codes leave four waves per SIMD)
     if (M >= 2 && bits <= 3 && group_size == 128 && row_blocks >= 1024) shape = 6;
