@@ -154,12 +154,20 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // and at 8 (57344 x 8192, 4 bits: 1728 against 1902 us).
       const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
       const bool g32zp = group_size == 32 && zp;
+      const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
+      const bool fits_192 = !(bf16 && (bits == 6 || group_size == 32)) && !(bits == 6 && g32zp);
       if (bits == 6 || bf16 || g32zp) {
-        const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
         const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
         const double t_128 = (double)((wgs_128 + 511) / 512);
-        const bool fits_192 = !(bf16 && (bits == 6 || group_size == 32)) && !(bits == 6 && g32zp);
         p->cfg = t_192 < t_128 && fits_192 ? 9 : 3;
+      } else if (wgs_192 <= 512 && fits_192) {
+        // Fewer than 512 of the 128 x 256 tiles leave half of the CUs with one workgroup where the
+        // kernel is built for two; 128 x 192 tiles that still fit one round of 512 spread the same
+        // rows over more of the slots (M = 2048, 4 bits: 6144 x 4096 92 against 98 us, 5120 x 4096 83
+        // against 91, 4608 x 3584 68 against 80; the same at 2, 3 and 8 bits).  Past 512 of them a
+        // second round starts and the 128 x 256 tile is ahead again (6144 x 4096, M = 2560: 139
+        // against 108 us).
+        p->cfg = 9;
       }
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X

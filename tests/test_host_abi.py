@@ -203,6 +203,17 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
 
 
+def test_planner_takes_192_row_tiles_where_they_fill_one_round_better():
+    # 6144 rows at M = 2048: 384 tiles of 128 x 256 leave half the CUs with one workgroup, 512 tiles
+    # of 128 x 192 fill every slot; past 512 of them the wide tile is back
+    for bits in (2, 3, 4, 8):
+        assert _lib.describe_plan(bits, 128, 6144, 4096, 2048, True).endswith("cfg9")
+    assert _lib.describe_plan(4, 32, 6144, 4096, 2048, False).endswith("cfg9")
+    assert _lib.describe_plan(4, -1, 5120, 4096, 2048, True).endswith("cfg9")
+    assert _lib.describe_plan(4, 128, 6144, 4096, 2560, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 7168, 4096, 2048, True).endswith("cfg0")
+
+
 def test_planner_takes_the_staged_tile_where_ring_tiles_would_sit_one_per_cu():
     assert _lib.describe_plan(4, 128, 8192, 8192, 512, True).endswith("cfg2")
     assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).endswith("cfg2")
