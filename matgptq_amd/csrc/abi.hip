@@ -172,18 +172,20 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
       // (4 bits, Llama-3-8B and 70B layers, M = 17 .. 1024), in microseconds:
-      //   128 x 128 tile  1.33 per K tile, up to 1.5 times that as a second workgroup joins a CU,
+      //   128 x 128 tile  1.55 per K tile, up to 2.0 as a second workgroup joins a CU,
       //                   proportionally more beyond the 512 resident slots;
-      //   32 x 128 tile   0.95 per K tile, proportionally more beyond 512 workgroups;
-      //   mid-batch kernel with 32 or 64 batch rows per workgroup: 2 + rounds x K tiles x
-      //                   (0.12 + 0.016 R MB), one workgroup per CU and round when its registers or
-      //                   LDS allow no second one (R = 4 or MB = 4), else two.
+      //   32 x 128 tile   0.95 per K tile and round of 512 workgroups, a last partial round
+      //                   counting as 0.35 of one at least;
+      //   mid-batch kernel with 32 or 64 batch rows per workgroup: 2 + rounds x (3.5 + K tiles x
+      //                   0.85 (0.12 + 0.016 R MB)), one workgroup per CU and round when its registers
+      //                   or LDS allow no second one (R = 4 or MB = 4), else two.
       const double kt = (double)k_tiles;
       const int64_t wgs_128 = ((N + 127) / 128) * ((M + 127) / 128);
       const int64_t wgs_32 = ((N + 127) / 128) * ((M + 31) / 32);
       const double second = wgs_128 <= 256 ? 0.0 : wgs_128 >= 512 ? 1.0 : (double)(wgs_128 - 256) / 256.0;
-      const double t_128 = 1.33 * kt * (1.0 + 0.5 * second) * (wgs_128 > 512 ? (double)wgs_128 / 512.0 : 1.0);
-      const double t_32 = 0.95 * kt * (wgs_32 > 512 ? (double)wgs_32 / 512.0 : 1.0);
+      const double t_128 = kt * (1.55 + 0.45 * second) * (wgs_128 > 512 ? (double)wgs_128 / 512.0 : 1.0);
+      const double rest_32 = (double)(wgs_32 % 512) / 512.0;
+      const double t_32 = 0.95 * kt * (wgs_32 <= 512 ? 1.0 : (double)(wgs_32 / 512) + (rest_32 == 0.0 ? 0.0 : rest_32 < 0.35 ? 0.35 : rest_32));
       p->cfg = t_128 < t_32 ? 3 : 4;
       // Where the 128 x 128 ring tiles would sit one per CU (it is built for two, whose waves cover
       // each other's waits), the staged 64 x 256 tile - twice the row blocks per dequantised
@@ -195,12 +197,30 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
           !(flags & MATGPTQ_FLAG_BF16))
         p->cfg = 2;
       double best = t_128 < t_32 ? t_128 : t_32;
+      // Ring tiles that sit one per CU run K in two halves inside a workgroup of eight waves (two
+      // per SIMD, as two workgroups would bring): 128 x 128 while those tiles number at most the
+      // CUs, 3 us + 1.0 .. 1.12 per K tile (M = 512: 8192 x 8192 73 against 87 us on the staged
+      // 64 x 256 tile, 8192 x 28672 249 against 298; 4096 x 4096 at M = 1024 40 against 48); 128 x 256 where
+      // only these number at most the CUs, 5 us + 1.4 .. 1.65 per K tile (8192 x 8192 at M = 1024 111
+      // against 125 us on 128 x 128 tiles two per CU, 8192 x 28672 366 against 440), for the formats
+      // whose registers fit that tile.
+      const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
+      if (wgs_128 <= 256) {
+        const double t = 3.0 + kt * (1.0 + 0.12 * (double)wgs_128 / 256.0);
+        if (t < best) { best = t; p->cfg = 10; }
+      } else if (wgs_big <= 256 && bits != 6 && !bf16 && !(group_size == 32 && zp)) {
+        const double t = 5.0 + kt * (wgs_big > 192 ? 1.65 : 1.4);
+        if (t < best) { best = t; p->cfg = 11; }
+      }
       for (int mb = 2; mb <= (M > 32 ? 4 : 2); mb <<= 1) {
         const int64_t m_tiles = (M + 16 * mb - 1) / (16 * mb);
         const int r = mid_rows(m_tiles);
         const int64_t wgs = (int64_t)((row_blocks + r - 1) / r) * m_tiles;
         const int64_t slots = 256 * (mb == 4 || r == 4 ? 1 : 2);
-        const double t = 2.0 + (double)((wgs + slots - 1) / slots) * kt * (0.12 + 0.016 * r * mb);
+        // (8-bit codes: twice the loads per weight of 4-bit ones, and two row blocks per workgroup at
+        // most; measured 1.6 times the cost per tile: 4096 x 14336 at M = 384 105 us)
+        const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (bits == 8 ? 1.6 : 1.0);
+        const double t = 2.0 + (double)((wgs + slots - 1) / slots) * (3.5 + kt * per_tile);
         if (t < best) {
           best = t;
           p->skinny = true;
@@ -275,7 +295,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       R = 1 << ((variant - 80) % 3);
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
-      if (variant - 64 > 9) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 11) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 64;

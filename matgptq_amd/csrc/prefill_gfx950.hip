@@ -13,7 +13,10 @@
 //    through registers: buffer_load ... lds copies them into a ring of four unpadded LDS
 //    buffers of 64 columns, three half tiles ahead, with an XOR swizzle of the 16-byte chunks
 //    against bank conflicts and hand-counted vmcnt waits in front of the workgroup barriers.
-//    One wave dequantises while the other wave of the SIMD multiplies;
+//    One wave dequantises while the other wave of the SIMD multiplies.  Where such tiles number
+//    no more than the CUs (batches of a few hundred rows), a workgroup of eight waves runs K in
+//    two halves on one tile, each group of four waves with a ring of its own, and adds the two
+//    sets of sums through LDS at the end: two waves per SIMD again, without a second workgroup;
 //  * the other tiles stage the activations through registers into two padded LDS buffers
 //    (global loads eight 32-column steps ahead, four for the largest tile) and pipeline inside
 //    a wave: while the matrix cores work on one 32-column step, the vector ALU dequantises the
@@ -92,10 +95,14 @@ __device__ __forceinline__ void refill_octet(BufRsrc rs, uint32_t tile_off, int 
 
 // One workgroup tile: activation rows [mtile * 16 MT, +16 MT) x the weight rows of the row blocks
 // rb_base + [nt * 4 RBW, +4 RBW), where lid = nt * m_tiles + mtile.  `lds` is the workgroup's
-// LDS (prefill_lds_halves(RBW, MT) halves, 16-byte aligned).
-template <int BITS, int GROUP, bool ZP, int RBW, int MT>
+// LDS (KS * prefill_lds_halves(RBW, MT) halves, 16-byte aligned).
+// KS = 2 (ring tiles only): a workgroup of eight waves, two groups of four that each walk one
+// half of K on the same tile with a ring of their own, so that a layer whose tiles number no more
+// than the CUs still runs two waves per SIMD; the second group's sums pass through LDS at the end.
+template <int BITS, int GROUP, bool ZP, int RBW, int MT, int KS = 1>
 __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_tiles, int rb_base,
                                              _Float16* lds) {
+  static_assert(KS == 1 || (KS == 2 && prefill_lean(RBW, MT)), "K is split inside the ring tiles only");
   constexpr int TM = 16 * MT;
   constexpr int GPT = GROUP == 32 ? 4 : 1;
   constexpr int XCHUNKS = TM * (kXs / 8) / 256;  // 16-byte chunks per thread per stage
@@ -105,7 +112,15 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile offsets stay scalar
+  const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile offsets stay scalar
+  const int wave = KS == 1 ? wave_wg : (wave_wg & 3);  // within its group of four
+  const int grp = KS == 1 ? 0 : (wave_wg >> 2);
+  // K tiles [k_lo, k_hi) in kt_n trips (the same count for both groups: they share the barriers; a
+  // tile beyond k_hi reads as zeros)
+  const int kt_n = KS == 1 ? a.k_tiles : (a.k_tiles + 1) / 2;
+  const int k_lo = grp * kt_n;
+  const int k_hi = KS == 1 || grp == 1 ? a.k_tiles : kt_n;
+  lds += grp * prefill_lds_halves(RBW, MT);
   const int r16 = lane & 15;
   const int q = lane >> 4;
 
@@ -136,11 +151,12 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
   // Branch-free loads: a tile beyond K, or a row block beyond N, is read through a
   // descriptor of zero length (every lane out of range: zeros come back, nothing is fetched).
   auto load_weights = [&](uint32_t (&w)[RBW][BITS], uint32_t (&s)[RBW][GPT], uint32_t (&z)[RBW][GPT],
-                          int kb) {
+                          int trip) {
+    const int kb = trip + k_lo;
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
       const int rb = rb_first + rr;
-      const bool valid = rb < a.row_blocks && kb < a.k_tiles;
+      const bool valid = rb < a.row_blocks && kb < k_hi;
       const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
       const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
       const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
@@ -271,8 +287,9 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       const uint32_t m = (uint32_t)(m0 + r);
       dma_voff[i] = m < (uint32_t)a.M ? (m * (uint32_t)a.K + c * 8) * 2u : x_bytes;
     }
-    auto dma = [&](_Float16* ring, int ih) {  // half tile ih of the walk into `ring`
-      const bool valid = ih < 2 * a.k_tiles;
+    auto dma = [&](_Float16* ring, int step) {  // half tile `step` of the walk into `ring`
+      const int ih = step + 2 * k_lo;
+      const bool valid = ih < 2 * k_hi;
       const BufRsrc xres = make_rsrc(a.x, valid ? x_bytes : 0u);
 #pragma unroll
       for (int i = 0; i < 4; i++)
@@ -347,22 +364,24 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       constexpr int r0 = RBW * refill_loads(BITS, 0), r1 = RBW * refill_loads(BITS, 1);
       constexpr int r2 = RBW * refill_loads(BITS, 2), r3 = RBW * refill_loads(BITS, 3);
       constexpr int kS = RBW * GPT * (ZP ? 2 : 1);
-      auto refill = [&](auto jtag, int kb) {  // octet J of tile kb into the one set of codes
+      auto refill = [&](auto jtag, int trip) {  // octet J of the tile of that trip into the one set of codes
         constexpr int J = decltype(jtag)::value;
+        const int kb = trip + k_lo;
 #pragma unroll
         for (int rr = 0; rr < RBW; rr++) {
           const int rb = rb_first + rr;
-          const bool valid = rb < a.row_blocks && kb < a.k_tiles;
+          const bool valid = rb < a.row_blocks && kb < k_hi;
           const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
           refill_octet<BITS, J>(wr, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, wcur[rr]);
         }
         __builtin_amdgcn_sched_barrier(0);
       };
-      auto load_aux = [&](uint32_t (&sv)[RBW][GPT], uint32_t (&zv)[RBW][GPT], int kb) {
+      auto load_aux = [&](uint32_t (&sv)[RBW][GPT], uint32_t (&zv)[RBW][GPT], int trip) {
+        const int kb = trip + k_lo;
 #pragma unroll
         for (int rr = 0; rr < RBW; rr++) {
           const int rb = rb_first + rr;
-          const bool valid = rb < a.row_blocks && kb < a.k_tiles;
+          const bool valid = rb < a.row_blocks && kb < k_hi;
           const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
           const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
 #pragma unroll
@@ -417,9 +436,9 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
         refill(J3{}, kb + 1);
         load_aux(sc, zc, kb + 2);  // this set is free now
       };
-      for (int kb = 0; kb < a.k_tiles; kb += 2) {
+      for (int kb = 0; kb < kt_n; kb += 2) {
         stile(kb, scur, zcur, ring0, ring1, ring2);
-        if (kb + 1 < a.k_tiles) stile(kb + 1, snxt, znxt, ring2, ring3, ring0);
+        if (kb + 1 < kt_n) stile(kb + 1, snxt, znxt, ring2, ring3, ring0);
       }
     } else {
     // buffer loads one load_weights() issues: the codes, then a scale (and a zero) per group
@@ -451,9 +470,9 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
         dstep(wc, sc, zc, J3{}, rn, 0);
         load_weights(wc, sc, zc, kb + 2);  // this set is free now
       };
-      for (int kb = 0; kb < a.k_tiles; kb += 2) {
+      for (int kb = 0; kb < kt_n; kb += 2) {
         dtile(kb, wcur, scur, zcur, ring0, ring1, ring2);
-        if (kb + 1 < a.k_tiles) dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
+        if (kb + 1 < kt_n) dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
       }
     }
   } else {
@@ -559,6 +578,32 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     __builtin_amdgcn_s_waitcnt(0);     // vmcnt(0) expcnt(0) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     _Float16* blk = lds + wave * (TM * ROWH);
+    if constexpr (KS == 2) {
+      // The second group hands its sums to the first as they lie in the registers (16 bytes per
+      // lane): those of its first H row blocks through its own ring, the others through the part of
+      // the first group's ring that wave `wave` of that group is about to use for its own output
+      // block, so no wave writes where another still reads.
+      constexpr int H = (RBW + 1) / 2;
+      static_assert((RBW - H) * MT * 64 * 16 <= TM * ROWH * 2 && 4 * H * MT * 64 * 16 <= prefill_lds_halves(RBW, MT) * 2,
+                    "the partial sums must fit the two rings");
+      _Float16* const lds0 = lds - grp * prefill_lds_halves(RBW, MT);
+      float4v* const p1 = reinterpret_cast<float4v*>(lds0 + prefill_lds_halves(RBW, MT)) + wave * (H * MT * 64) + lane;
+      float4v* const p0 = reinterpret_cast<float4v*>(lds0 + wave * (TM * ROWH)) + lane;
+      if (grp == 1) {
+#pragma unroll
+        for (int rr = 0; rr < RBW; rr++)
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++)
+            (rr < H ? p1[(rr * MT + mt) * 64] : p0[((rr - H) * MT + mt) * 64]) = acc[rr][mt];
+      }
+      __syncthreads();
+      if (grp == 1) return;
+#pragma unroll
+      for (int rr = 0; rr < RBW; rr++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+          acc[rr][mt] += rr < H ? p1[(rr * MT + mt) * 64] : p0[((rr - H) * MT + mt) * 64];
+    }
 #pragma unroll
     for (int rr = 0; rr < RBW; rr++) {
 #pragma unroll
@@ -619,6 +664,15 @@ prefill_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   prefill_body<BITS, GROUP, ZP, RBW, MT>(a, lid, m_tiles, 0, lds);
 }
 
+// A ring tile with K split over two groups of four waves (see prefill_body): one workgroup per
+// CU holds the eight waves that two workgroups of the plain kernel would bring.
+template <int BITS, int GROUP, bool ZP, int RBW, int MT>
+__global__ void __launch_bounds__(512, 2)
+prefill_split_kernel(const GemmArgs a, int m_tiles) {
+  __shared__ __align__(16) _Float16 lds[2 * prefill_lds_halves(RBW, MT)];
+  prefill_body<BITS, GROUP, ZP, RBW, MT, 2>(a, blockIdx.x, m_tiles, 0, lds);
+}
+
 // 128 x 256 tiles with a tail of 128 x 128 tiles.  The larger tile keeps 512 workgroups
 // resident (two per CU); when a layer gives it a whole number of such rounds plus a fraction,
 // that fraction would run as one more round at the full length of a tile.  Here the first
@@ -658,9 +712,20 @@ hipError_t launch_cfg(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <int GROUP, bool ZP, int RBW, int MT>
+hipError_t launch_split(const GemmArgs& a, hipStream_t stream) {
+  const int n_tiles = (a.row_blocks + 4 * RBW - 1) / (4 * RBW);
+  const int m_tiles = (a.M + 16 * MT - 1) / (16 * MT);
+  const dim3 grid(n_tiles * m_tiles), block(512);
+  hipLaunchKernelGGL((prefill_split_kernel<kBits, GROUP, ZP, RBW, MT>), grid, block, 0, stream, a, m_tiles);
+  return hipGetLastError();
+}
+
 template <int GROUP, bool ZP>
 hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
   switch (cfg) {
+    case 10: return launch_split<GROUP, ZP, 2, 8>(a, s);  // 128 x 128, K split in the workgroup
+    case 11: return launch_split<GROUP, ZP, 4, 8>(a, s);  // 128 x 256, K split in the workgroup
     case 0: return launch_cfg<GROUP, ZP, 4, 8>(a, s);   // 128 x 256
     case 1: return launch_cfg<GROUP, ZP, 8, 8>(a, s);   // 128 x 512
     case 2: return launch_cfg<GROUP, ZP, 4, 4>(a, s);   // 64 x 256

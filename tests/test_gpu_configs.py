@@ -62,6 +62,27 @@ def test_config4_prefill_full_size(name, plan):
     G.assert_close_to_reference(yr, ref, bound, f"70B {name} prefill")
 
 
+@pytest.mark.parametrize("name,m,plan", [("o", 512, "prefill b4 g128 zp1 cfg10"), ("o", 1024, "prefill b4 g128 zp1 cfg11"),
+                                         ("down", 500, "prefill b4 g128 zp1 cfg10"), ("down", 1000, "prefill b4 g128 zp1 cfg11")])
+def test_medium_batch_split_tiles_full_size(name, m, plan):
+    # batches of a few hundred rows on the Llama-3-70B layers with 8192 rows: the ring tiles with K
+    # split inside a workgroup of eight waves (down: 112 K tiles per group of waves; ragged M)
+    n, k = LLAMA70B[name]
+    assert _lib.describe_plan(4, 128, n, k, m, True) == plan
+    q, s, z = o.make_layer(n, k, 128, seed=17)
+    x = o.make_activations(m, k, seed=m)
+    packed = G.pack_device(q, 4, True)
+    sc, zr = G.reorder_device(s, n, k, 128), G.reorder_device(z, n, k, 128)
+    y = G.gemm(4, 128, n, k, G.to_dev(x), packed, sc, zr)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y.float()).all())
+    tiles = (m + 127) // 128
+    rows = np.array(sorted({min(t * 128 + (37 * t + 5) % 128, m - 1) for t in range(tiles)} | {0, m - 1}))
+    yr = y[torch.from_numpy(rows).to(G.DEV)].cpu().numpy()
+    ref, bound = G.oracle_product_in_chunks(q, s, z, 4, 128, x[rows])
+    G.assert_close_to_reference(yr, ref, bound, f"70B {name} M={m}")
+
+
 @pytest.mark.parametrize("m", (1, 2, 4))
 def test_llama3_70b_down_decode_full_size(m):
     # 224 K tiles per row block: sixteen waves walk three and a half rounds

@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(10))
+@pytest.mark.parametrize("cfg", range(12))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -130,6 +130,45 @@ def test_prefill_ring_tile_every_format(b, g, zp):
         y = lay.run(x, flags=1 | (64 << 8))
         G.assert_close_to_oracle(y, x, lay.w, f"ring tile b={b} g={g} zp={zp}")
     assert _lib.describe_plan(b, g, n, k, m, zp, 1 | (64 << 8)).endswith("cfg0")
+
+
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("g", GROUPS)
+@pytest.mark.parametrize("b", BITS)
+def test_prefill_split_tiles_every_format(b, g, zp):
+    # K in two halves inside a workgroup of eight waves, each group with a ring of its own and
+    # the same hand-counted waits; the second group's sums cross LDS at the end.  Seven K tiles
+    # (the second group walks one tile fewer), ragged M and N; both tile widths.
+    n, k, m = 304, 128 * 7, 200
+    lay = G.Layer(n, k, b, g, seed=29 * b + (g & 7), zero_points=zp)
+    x = o.make_activations(m, k, seed=b + 2)
+    for cfg in (10, 11):
+        flags = 1 | ((64 + cfg) << 8)
+        for _ in range(2):
+            G.assert_close_to_oracle(lay.run(x, flags=flags), x, lay.w, f"split tile cfg{cfg} b={b} g={g} zp={zp}")
+        assert _lib.describe_plan(b, g, n, k, m, zp, flags).endswith(f"cfg{cfg}")
+
+
+@pytest.mark.parametrize("k_tiles", (1, 2, 3, 10))
+@pytest.mark.parametrize("cfg", (10, 11))
+def test_prefill_split_tiles_short_and_even_walks(cfg, k_tiles):
+    # one K tile leaves the second group with nothing but zeros; two give each group a single trip
+    n, k, m = 528, 128 * k_tiles, 130
+    lay = G.Layer(n, k, 4, 128, seed=k_tiles)
+    x = o.make_activations(m, k, seed=cfg)
+    G.assert_close_to_oracle(lay.run(x, flags=1 | ((64 + cfg) << 8)), x, lay.w, f"split cfg{cfg} {k_tiles} K tiles")
+
+
+def test_prefill_split_tile_agrees_with_the_plain_tile_closely():
+    # the same products in the same order within each half of K; the two halves are added in fp32
+    n, k, m = 1024, 4096, 256
+    lay = G.Layer(n, k, 4, 128, seed=8)
+    x = o.make_activations(m, k, seed=9)
+    plain = lay.run(x, flags=1 | (67 << 8)).astype(np.float64)
+    for cfg in (10, 11):
+        y = lay.run(x, flags=1 | ((64 + cfg) << 8)).astype(np.float64)
+        assert np.max(np.abs(y - plain)) <= 2.0 ** -9 * np.max(np.abs(plain))
+        assert np.mean(y == plain) > 0.9
 
 
 @pytest.mark.parametrize("zp", (False, True))
@@ -415,7 +454,8 @@ def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
     # The prefill kernel multiplies bf16 by bf16 on the matrix cores.  With the identity as
     # activations every output is one weight (plus exact zeros), so the result must be
     # dequantize() on bfloat16 tensors, bit for bit (integer zero points: one rounding on both
-    # sides).  Ring tiles 128 x 256, 128 x 128, 128 x 192, the tail split and a staged tile.
+    # sides).  Ring tiles 128 x 256, 128 x 128, 128 x 192, the tail split, a staged tile and the two
+    # tiles that split K inside the workgroup.
     n, k, g = 304, 256, 128
     q, s16, z16 = o.make_layer(n, k, g, seed=300 + b, symmetric=not zp)
     s = o.round_to_bf16(s16.astype(np.float32))
@@ -423,12 +463,13 @@ def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
     x = np.eye(k, dtype=np.float32)
     pk = G.pack_device(q, b, True)
     w = o.dequantize_bf16(q, s, z, b, g)
-    for cfg in (64, 67, 73, 72, 66):
+    for cfg in (64, 67, 73, 72, 66, 74, 75):
         y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | (cfg << 8))
         assert np.array_equal(y, w.T), (b, zp, cfg)
 
 
-@pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8), 3 | (67 << 8), 3 | (72 << 8), 3 | (73 << 8)))
+@pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8), 3 | (67 << 8), 3 | (72 << 8), 3 | (73 << 8), 3 | (74 << 8),
+                                   3 | (75 << 8)))
 def test_bf16_prefill_large_tiles(flags):
     # default choice for a large batch, and the ring and largest tiles forced
     n, k, m, b, g = 2048, 1024, 2048, 4, 128

@@ -214,13 +214,22 @@ def test_planner_takes_192_row_tiles_where_they_fill_one_round_better():
     assert _lib.describe_plan(4, 128, 7168, 4096, 2048, True).endswith("cfg0")
 
 
-def test_planner_takes_the_staged_tile_where_ring_tiles_would_sit_one_per_cu():
-    assert _lib.describe_plan(4, 128, 8192, 8192, 512, True).endswith("cfg2")
-    assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).endswith("cfg2")
-    assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True).endswith("cfg3")    # two ring tiles per CU
-    assert _lib.describe_plan(4, 128, 10240, 8192, 512, True).endswith("cfg3")
-    assert _lib.describe_plan(4, 32, 8192, 8192, 512, True).endswith("cfg3")      # group 32: registers
-    assert _lib.describe_plan(4, 128, 8192, 8192, 512, True, 3).endswith("cfg3")  # bf16 storage
+def test_planner_splits_k_in_the_workgroup_where_ring_tiles_would_sit_one_per_cu():
+    # 128 x 128 tiles that number at most the CUs: eight waves per workgroup, K in two halves
+    assert _lib.describe_plan(4, 128, 8192, 8192, 512, True).endswith("cfg10")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).endswith("cfg10")
+    assert _lib.describe_plan(4, 32, 8192, 8192, 512, True).endswith("cfg10")      # every format fits it
+    assert _lib.describe_plan(4, 128, 8192, 8192, 512, True, 3).endswith("cfg10")  # bf16 storage too
+    # more of those than CUs but at most as many 128 x 256 tiles: the wide tile, split
+    assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True).endswith("cfg11")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 512, True).endswith("cfg11")
+    assert _lib.describe_plan(8, 128, 8192, 8192, 1024, True).endswith("cfg11")
+    assert _lib.describe_plan(6, 128, 8192, 8192, 1024, True).endswith("cfg3")     # 6 bits: registers
+    assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True, 3).endswith("cfg3")  # bf16 likewise
+    # short K walks as well, down to where the small staged tile fits one round
+    assert _lib.describe_plan(4, 128, 4096, 2048, 1024, True).endswith("cfg10")
+    assert _lib.describe_plan(4, 128, 4096, 1024, 1024, True).endswith("cfg10")
+    assert _lib.describe_plan(4, 128, 4096, 1024, 512, True).endswith("cfg4")
 
 
 def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
