@@ -475,6 +475,26 @@ def main() -> int:
             del wd
             torch.cuda.empty_cache()
         extra["speedup_over_dense_fp16"] = speed
+        # ------------------------------------------------ batches of a few hundred rows
+        # (chunked prefill): the Llama-3-70B layers at 4 bits, zero-point form, beside the dense
+        # fp16 product on the same GPU; graphs of five launches, median of five replays
+        medium = {}
+        for name, (n, k) in LLAMA3_70B.items():
+            packed = make_ring(n, k, 4, 1)[0]
+            sc, zr = make_aux(n, k)
+            wd = (torch.randn(n, k, device=dev, generator=g) * 0.02).to(torch.float16)
+            for m in (128, 256, 512, 1024):
+                xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+                ym = torch.empty(m, n, dtype=torch.float16, device=dev)
+                t = timed_graph(lambda: [launch(4, n, k, xm, packed, sc, zr, ym) for _ in range(5)]) / 5
+                t_dense = timed_graph(lambda: [torch.nn.functional.linear(xm, wd) for _ in range(5)]) / 5
+                medium[f"{name}_M{m}"] = {"us": round(t * 1e6, 1), "dense_us": round(t_dense * 1e6, 1),
+                                          "speedup": round(t_dense / t, 2),
+                                          "TFLOPs": round(2.0 * m * n * k / t / 1e12, 1),
+                                          "kernel": _lib.describe_plan(4, GROUP, n, k, m, True)}
+            del packed, wd
+            torch.cuda.empty_cache()
+        extra["medium_batch_llama3_70b_b4"] = medium
         # ---------------------------------------------------------- load time
         # What process_weights_after_loading costs per layer (gate_up of Llama-3-8B, 117 M master
         # codes already in HBM): slice + pack in one kernel (reads 1 byte per code, writes b/8),
