@@ -82,11 +82,13 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
-    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill", "midbatch"),
+    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill", "midbatch", "medium"),
                     help="for rocprofv3 --pmc runs.  decode: launch only the dominant kernel over the ring of "
                          "weight copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's "
                          "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer.  "
-                         "midbatch: launch only the mid-batch kernel, 4096->4096 at M=64 and 14336->4096 at M=16")
+                         "midbatch: launch only the mid-batch kernel, 4096->4096 at M=64 and 14336->4096 at M=16.  "
+                         "medium: launch only the ring tiles that split K inside the workgroup, 8192->8192 at "
+                         "M=512 and M=1024")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -123,9 +125,11 @@ def main() -> int:
         zeros = torch.randint(0, 256, (groups,), device=dev, generator=g).to(torch.float16)
         return scales, zeros
 
-    def timed_graph(build, reps=5):
+    def timed_graph(build, reps=5, settle_ms=0.0):
         """Captures `build()` (launches on `stream`) into a HIP graph; returns the median
-        replay time in seconds over `reps` replays, measured with events on `stream`."""
+        replay time in seconds over `reps` replays, measured with events on `stream`.
+        `settle_ms`: keep replaying, untimed, for that long first (the clocks take some
+        milliseconds to settle after the allocation and random fill of a new ring of weights)."""
         with torch.cuda.stream(stream):
             build()  # eager warm-up of every kernel in the graph
             stream.synchronize()
@@ -134,6 +138,10 @@ def main() -> int:
                 build()
             graph.replay()
             stream.synchronize()
+            t_end = time.perf_counter() + settle_ms * 1e-3
+            while time.perf_counter() < t_end:
+                graph.replay()
+                stream.synchronize()
             times = []
             for _ in range(reps):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -156,6 +164,21 @@ def main() -> int:
                 launch(bits, n, k, x, packed, sc, zr, y)
             stream.synchronize()
         print(json.dumps({"counter_pass": _lib.describe_plan(bits, GROUP, n, k, 2048, True), "launches": 6}))
+        return 0
+    if args.counter_pass == "medium":
+        n, k = LLAMA3_70B["o"]
+        packed = make_ring(n, k, bits, 1)[0]
+        sc, zr = make_aux(n, k)
+        plans = []
+        for m in (512, 1024):
+            x = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+            y = torch.empty(m, n, dtype=torch.float16, device=dev)
+            with torch.cuda.stream(stream):
+                for _ in range(6):
+                    launch(bits, n, k, x, packed, sc, zr, y)
+                stream.synchronize()
+            plans.append(f"M={m}: " + _lib.describe_plan(bits, GROUP, n, k, m, True))
+        print(json.dumps({"counter_pass": plans, "launches_each": 6}))
         return 0
     if args.counter_pass == "midbatch":
         plans = []
@@ -290,7 +313,7 @@ def main() -> int:
                 for zp in (True, False):
                     t = timed_graph(lambda: [launch(b, n, k, xs[name], ring[i % cp], aux[name][0],
                                                     aux[name][1] if zp else None, ys[name])
-                                             for i in range(reps)]) / reps
+                                             for i in range(reps)], settle_ms=0.0 if b == bits else 15.0) / reps
                     table[f"{name}_b{b}_{'zp' if zp else 'sym'}"] = {
                         "us": round(t * 1e6, 2),
                         "weight_GBps": round(wbytes / t / 1e9, 1),
