@@ -177,15 +177,16 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       //   32 x 128 tile   0.95 per K tile and round of 512 workgroups, a last partial round
       //                   counting as 0.35 of one at least;
       //   mid-batch kernel with 32 or 64 batch rows per workgroup: 2 + rounds x (3.5 + K tiles x
-      //                   0.85 (0.12 + 0.016 R MB)), one workgroup per CU and round when its registers
-      //                   or LDS allow no second one (R = 4 or MB = 4), else two.
+      //                   0.85 (0.12 + 0.016 R MB)), one workgroup per CU and round.
       const double kt = (double)k_tiles;
       const int64_t wgs_128 = ((N + 127) / 128) * ((M + 127) / 128);
       const int64_t wgs_32 = ((N + 127) / 128) * ((M + 31) / 32);
       const double second = wgs_128 <= 256 ? 0.0 : wgs_128 >= 512 ? 1.0 : (double)(wgs_128 - 256) / 256.0;
       const double t_128 = kt * (1.55 + 0.45 * second) * (wgs_128 > 512 ? (double)wgs_128 / 512.0 : 1.0);
       const double rest_32 = (double)(wgs_32 % 512) / 512.0;
-      const double t_32 = 0.95 * kt * (wgs_32 <= 512 ? 1.0 : (double)(wgs_32 / 512) + (rest_32 == 0.0 ? 0.0 : rest_32 < 0.35 ? 0.35 : rest_32));
+      // (bf16 storage 1.2 times that, group size 32 - four scales and zeros per tile - 1.4 times)
+      const double t_32 = 0.95 * ((flags & MATGPTQ_FLAG_BF16) ? 1.2 : 1.0) * (group_size == 32 ? 1.4 : 1.0) * kt *
+                          (wgs_32 <= 512 ? 1.0 : (double)(wgs_32 / 512) + (rest_32 == 0.0 ? 0.0 : rest_32 < 0.35 ? 0.35 : rest_32));
       p->cfg = t_128 < t_32 ? 3 : 4;
       // Where the 128 x 128 ring tiles would sit one per CU (it is built for two, whose waves cover
       // each other's waits), the staged 64 x 256 tile - twice the row blocks per dequantised
@@ -216,10 +217,13 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         const int64_t m_tiles = (M + 16 * mb - 1) / (16 * mb);
         const int r = mid_rows(m_tiles);
         const int64_t wgs = (int64_t)((row_blocks + r - 1) / r) * m_tiles;
-        const int64_t slots = 256 * (mb == 4 || r == 4 ? 1 : 2);
-        // (8-bit codes: twice the loads per weight of 4-bit ones, and two row blocks per workgroup at
-        // most; measured 1.6 times the cost per tile: 4096 x 14336 at M = 384 105 us)
-        const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (bits == 8 ? 1.6 : 1.0);
+        // One workgroup per CU and round.  (With 32 batch rows and at most two row blocks a second
+        // one fits, but two together take 1.6 times as long as one: 0.8 of the cost per tile each.)
+        // 8-bit codes cost 1.1 times as much per tile, bf16 storage (weights formed in fp32) 1.45
+        // times: 8192 x 8192, group 32, M = 256, 64 batch rows per workgroup: 73 us fp16, 113 us bf16.
+        const int64_t slots = 256;
+        const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (mb == 2 && r <= 2 ? 0.8 : 1.0) *
+                                (bits == 8 ? 1.1 : 1.0) * (bf16 ? 1.45 : 1.0);
         const double t = 2.0 + (double)((wgs + slots - 1) / slots) * (3.5 + kt * per_tile);
         if (t < best) {
           best = t;

@@ -188,7 +188,7 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(4, 32, 4096, 14336, 5, True).startswith("midbatch")
     assert _lib.describe_plan(3, 32, 16, 1024, 17).startswith("midbatch")
     assert _lib.describe_plan(4, 128, 4096, 4096, 128, True) == "midbatch b4 g128 zp1 R4 mb2"
-    assert _lib.describe_plan(8, 128, 4096, 4096, 128, True) == "midbatch b8 g128 zp1 R2 mb2"
+    assert _lib.describe_plan(8, 128, 4096, 4096, 128, True) == "midbatch b8 g128 zp1 R2 mb4"
     assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).startswith("prefill")
     assert _lib.describe_plan(4, 128, 4096, 4096, 16, True, 1 | (1 << 8)).startswith("decode")
 
