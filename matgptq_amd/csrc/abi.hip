@@ -219,11 +219,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         const int64_t wgs = (int64_t)((row_blocks + r - 1) / r) * m_tiles;
         // One workgroup per CU and round.  (With 32 batch rows and at most two row blocks a second
         // one fits, but two together take 1.6 times as long as one: 0.8 of the cost per tile each.)
-        // 8-bit codes cost 1.1 times as much per tile, bf16 storage (weights formed in fp32) 1.45
-        // times: 8192 x 8192, group 32, M = 256, 64 batch rows per workgroup: 73 us fp16, 113 us bf16.
+        // 8-bit codes cost 1.1 times as much per tile, bf16 storage (weights formed in fp32) 1.12
+        // times: 8192 x 8192, M = 256, 64 batch rows per workgroup: 49.5 us fp16, 53.8 us bf16.
         const int64_t slots = 256;
         const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (mb == 2 && r <= 2 ? 0.8 : 1.0) *
-                                (bits == 8 ? 1.1 : 1.0) * (bf16 ? 1.45 : 1.0);
+                                (bits == 8 ? 1.1 : 1.0) * (bf16 ? 1.12 : 1.0);
         const double t = 2.0 + (double)((wgs + slots - 1) / slots) * (3.5 + kt * per_tile);
         if (t < best) {
           best = t;

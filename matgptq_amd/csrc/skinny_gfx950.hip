@@ -11,7 +11,8 @@
 //    wave w takes the K tiles w, w + 8, ... of those rows, so a layer with N / (16 R) x M / (16 MB)
 //    output tiles still runs eight times as many waves, each with a short K walk;
 //  * each wave dequantises its tiles from registers into the 16x32 MFMA operand (the same
-//    arithmetic as the large-batch kernel).  No two waves of a workgroup read the same
+//    arithmetic as the large-batch kernel: fp16 weights times fp16 activations, or bf16 weights,
+//    formed in fp32 and rounded once, times the bf16 activations as stored).  No two waves of a workgroup read the same
 //    activations, so every wave stages its own: buffer_load ... lds copies the 16*MB x 128
 //    activations of a tile from global memory straight into the wave's private LDS buffer,
 //    256 contiguous bytes per 16 lanes (an operand read straight from global memory
@@ -91,6 +92,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     for (int i = 0; i < MB; i++) acc[rr][i] = float4v{0.f, 0.f, 0.f, 0.f};
 
   const UnpackConsts<BITS> kc_unpack;
+  const float kc_zero = __uint_as_float(opaque_vgpr(0u));  // a zero the optimiser cannot see through
   // codes, scales and zeros of the tile in use and of the next one; scales and zeros stay as
   // loaded and are converted where they are used
   uint32_t wr[NS][R][BITS], sr[NS][R][GPT], zr[NS][R][GPT];
@@ -147,20 +149,24 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
       const int gg = GROUP == 32 ? J : 0;
-      // fp16 storage: scale * 2^(8-b) and scale * (zero - 128);
-      // bf16 storage: scale * 2^8 and (zero - 128) * 2^-8, converted through fp32
-      _Float16 s1, z1 = (_Float16)0.f;
       if constexpr (kBf16) {
-        s1 = (_Float16)(bf16_bits_to_float(s[rr][gg]) * 256.0f);
-        if constexpr (ZP) z1 = (_Float16)((bf16_bits_to_float(z[rr][gg]) - 128.0f) * (1.0f / 256.0f));
+        // bf16 storage: the activations go to the bf16 matrix instruction as stored; the weights
+        // are formed in fp32 from scale * 2^(8-b) and scale * (zero - 128) and rounded to bf16 once
+        const float s0 = bf16_bits_to_float(s[rr][gg]);
+        const float sm = s0 * (float)(1 << (8 - BITS));
+        float sz = kc_zero;
+        if constexpr (ZP) sz = s0 * (bf16_bits_to_float(z[rr][gg]) - 128.0f);
+        dequant_octet_bf16<BITS, J>(w[rr], kc_unpack, sm, sz, aw[rr]);
       } else {
+        // fp16 storage: scale * 2^(8-b) and scale * (zero - 128)
         const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)s[rr][gg]);
-        s1 = (_Float16)((float)s0 * (float)(1 << (8 - BITS)));  // scale * m
+        const _Float16 s1 = (_Float16)((float)s0 * (float)(1 << (8 - BITS)));  // scale * m
+        _Float16 z1 = (_Float16)0.f;
         if constexpr (ZP) z1 = s0 * (__builtin_bit_cast(_Float16, (uint16_t)z[rr][gg]) - (_Float16)128.0f);
+        const half2v sc = {s1, s1};
+        const half2v zr = {z1, z1};
+        dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
       }
-      const half2v sc = {s1, s1};
-      const half2v zr = {z1, z1};
-      dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
     }
   };
 
@@ -191,10 +197,14 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
         dequant_step(aw, wr[B], sr[B], zr[B], jtag);
 #pragma unroll
         for (int i = 0; i < MB; i++) {
-          const half8 b = storage8_to_half8(xf[J][i]);
 #pragma unroll
-          for (int rr = 0; rr < R; rr++)
-            acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, b, acc[rr][i], 0, 0, 0);
+          for (int rr = 0; rr < R; rr++) {
+            if constexpr (kBf16)
+              acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, aw[rr].h),
+                                                                  __builtin_bit_cast(bf16x8, xf[J][i]), acc[rr][i], 0, 0, 0);
+            else
+              acc[rr][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aw[rr].h, xf[J][i], acc[rr][i], 0, 0, 0);
+          }
         }
       };
       one(std::integral_constant<int, 0>{});
