@@ -234,15 +234,16 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       }
     }
   } else if (flavour == 0 && M > kGemvMaxM &&
-             (row_blocks < 1024 || r_max == 4 || (group_size == 32 && bits <= 4))) {
+             !(bits == 8 && group_size != 32 && !(flags & MATGPTQ_FLAG_BF16) && row_blocks >= 1024)) {
     // Five to sixteen batch rows (one to four go to the gemv kernel below): every decode
     // workgroup stages the whole batch of activations (scaled copies, written by the vector
     // ALU), which grows with M and K, while the mid-batch kernel copies them into LDS
     // asynchronously.  Measured on MI355X (Llama-3-8B layers, 2, 4 and 8 bits, M = 5 .. 16, weights
     // cold): the mid-batch kernel wins everywhere (M = 7, 4 bits: 4096 x 4096 5.4 against 7.3 us,
-    // 6144 x 4096 6.1 against 8.5, 28672 x 4096 15.8 against 20.4) except on layers with many
-    // rows where it may take two row blocks only: 8 bits (28672 x 4096: 24.8 against 23.7 us), and
-    // group size 32 above 4 bits (at 4 bits, M = 8: 20.9 against 28.2 us; 8 bits tie at 29).
+    // 6144 x 4096 6.1 against 8.5, 28672 x 4096 15.8 against 20.4; group size 32 at 6 and 8 bits,
+    // M = 8: 23.3 and 23.7 against 33.8 and 29.0; bf16 storage at 8 bits 21.7 against 25.2) except at
+    // 8 bits on fp16 storage with one scale per tile or row, on layers with many rows, where it
+    // may take two row blocks only (28672 x 4096: 24.8 against 23.7 us).
     p->decode = false;
     p->skinny = true;
     p->mb = 1;

@@ -166,12 +166,15 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(3, 128, 28672, 4096, 4, True) == "gemv b3 g128 zp1 T4 R4 W8 pad0"
     assert _lib.describe_plan(3, 128, 6144, 4096, 4, True) == "gemv b3 g128 zp1 T4 R2 W8 pad0"
     assert _lib.describe_plan(4, 32, 4096, 4096, 5).startswith(("decode", "midbatch"))
-    # five to sixteen rows: the mid-batch kernel, except on layers with many rows where it may take
-    # two row blocks only (8 bits; group size 32 above 4 bits)
+    # five to sixteen rows: the mid-batch kernel, except at 8 bits on fp16 storage with one scale per
+    # tile or row, on layers with many rows (two row blocks per workgroup only)
     assert _lib.describe_plan(4, 32, 28672, 4096, 8, True) == "midbatch b4 g32 zp1 R2 mb1"
     assert _lib.describe_plan(4, 32, 28672, 4096, 5, True) == "midbatch b4 g32 zp1 R2 mb1"
-    assert _lib.describe_plan(8, 32, 28672, 4096, 8, True).startswith("decode")
+    assert _lib.describe_plan(8, 32, 28672, 4096, 8, True) == "midbatch b8 g32 zp1 R2 mb1"
+    assert _lib.describe_plan(6, 32, 28672, 4096, 16, True) == "midbatch b6 g32 zp1 R2 mb1"
+    assert _lib.describe_plan(8, 128, 28672, 4096, 8, True, 3) == "midbatch b8 g128 zp1 R2 mb1"  # bf16
     assert _lib.describe_plan(8, 128, 28672, 4096, 5, True).startswith("decode")
+    assert _lib.describe_plan(8, -1, 28672, 4096, 16, False).startswith("decode")
     assert _lib.describe_plan(4, 128, 28672, 4096, 5, True) == "midbatch b4 g128 zp1 R4 mb1"
     assert _lib.describe_plan(8, 128, 4096, 4096, 5, True) == "midbatch b8 g128 zp1 R1 mb1"
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048).startswith("prefill")
