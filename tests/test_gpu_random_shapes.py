@@ -40,6 +40,28 @@ def test_random_problems_through_the_default_plan(seed):
         G.assert_regression_bound(y, x, lay.w, what)
 
 
+@pytest.mark.parametrize("seed", (20, 21))
+def test_random_larger_problems_through_the_default_plan(seed):
+    # a few thousand weight rows and batches of hundreds to two thousand rows: the ring tiles, the
+    # tiles that split K inside the workgroup and the larger mid-batch shapes; sampled batch rows
+    rng = np.random.default_rng(seed)
+    for it in range(10):
+        b = int(rng.choice(BITS))
+        g = int(rng.choice((128, 128, 32, -1)))
+        n = 16 * int(rng.choice((64, 100, 160, 256, 288, 384, 512)))
+        tiles = int(rng.choice((3, 8, 9, 16, 31, 32)))
+        k = 128 * tiles + (64 if g != 128 and rng.random() < 0.2 else 0)
+        m = int(rng.choice((130, 250, 384, 500, 512, 640, 777, 1024, 1100, 1536, 2048)))
+        zp = bool(rng.integers(0, 2))
+        lay = G.Layer(n, k, b, g, seed=1000 * seed + it, zero_points=zp)
+        x = o.make_activations(m, k, seed=it + m, outlier_frac=0.01)
+        what = f"b={b} g={g} N={n} K={k} M={m} zp={zp} [{_lib.describe_plan(b, g, n, k, m, zp)}]"
+        y = lay.run(x)
+        rows = np.unique(np.r_[0, m - 1, rng.integers(0, m, 22)])
+        G.assert_close_to_oracle(y[rows], x[rows], lay.w, what)
+        G.assert_regression_bound(y[rows], x[rows], lay.w, what)
+
+
 def _bf16_dev(a):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(G.DEV)
