@@ -128,7 +128,21 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     // once its workgroups fill more than half of the 512 resident slots (measured on MI355X,
     // Llama-3-8B and 70B layers).
     const int64_t wgs_big = ((N + 255) / 256) * ((M + 127) / 128);
-    if (wgs_big >= 288) {
+    // the 32 x 128 staged tile: 0.95 us per K tile and round of 512 workgroups, a last partial round
+    // counting as 0.35 of one at least (bf16 storage 1.2 times that, group size 32 - four scales and
+    // zeros per tile - 1.4 times)
+    const int64_t wgs_32 = ((N + 127) / 128) * ((M + 31) / 32);
+    const double rest_32 = (double)(wgs_32 % 512) / 512.0;
+    const double t_32 = 0.95 * ((flags & MATGPTQ_FLAG_BF16) ? 1.2 : 1.0) * (group_size == 32 ? 1.4 : 1.0) * (double)k_tiles *
+                        (wgs_32 <= 512 ? 1.0 : (double)(wgs_32 / 512) + (rest_32 == 0.0 ? 0.0 : rest_32 < 0.35 ? 0.35 : rest_32));
+    // A layer with very many rows fills the 128 x 256 tiles' slots at any batch size, but up to 64 batch
+    // rows those tiles are mostly padding: a round of them costs 11.5 us + 3.2 per K tile (128256 x 4096 at
+    // M = 32: 117 us, against 65 on the small tile).
+    const bool small_batch_many_rows =
+        M <= 64 && t_32 < (11.5 + 3.2 * (double)k_tiles) * (wgs_big > 512 ? (double)wgs_big / 512.0 : 1.0);
+    if (wgs_big >= 288 && small_batch_many_rows) {
+      p->cfg = 4;
+    } else if (wgs_big >= 288) {
       p->cfg = 0;
       // Whole rounds of 512 resident workgroups plus at most half a round: the rows of that
       // fraction go to 128 x 128 tiles, which run last, one per CU, in about a third of a
@@ -174,19 +188,13 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // (4 bits, Llama-3-8B and 70B layers, M = 17 .. 1024), in microseconds:
       //   128 x 128 tile  1.55 per K tile, up to 2.0 as a second workgroup joins a CU,
       //                   proportionally more beyond the 512 resident slots;
-      //   32 x 128 tile   0.95 per K tile and round of 512 workgroups, a last partial round
-      //                   counting as 0.35 of one at least;
+      //   32 x 128 tile   as above;
       //   mid-batch kernel with 32 or 64 batch rows per workgroup: 2 + rounds x (3.5 + K tiles x
       //                   0.85 (0.12 + 0.016 R MB)), one workgroup per CU and round.
       const double kt = (double)k_tiles;
       const int64_t wgs_128 = ((N + 127) / 128) * ((M + 127) / 128);
-      const int64_t wgs_32 = ((N + 127) / 128) * ((M + 31) / 32);
       const double second = wgs_128 <= 256 ? 0.0 : wgs_128 >= 512 ? 1.0 : (double)(wgs_128 - 256) / 256.0;
       const double t_128 = kt * (1.55 + 0.45 * second) * (wgs_128 > 512 ? (double)wgs_128 / 512.0 : 1.0);
-      const double rest_32 = (double)(wgs_32 % 512) / 512.0;
-      // (bf16 storage 1.2 times that, group size 32 - four scales and zeros per tile - 1.4 times)
-      const double t_32 = 0.95 * ((flags & MATGPTQ_FLAG_BF16) ? 1.2 : 1.0) * (group_size == 32 ? 1.4 : 1.0) * kt *
-                          (wgs_32 <= 512 ? 1.0 : (double)(wgs_32 / 512) + (rest_32 == 0.0 ? 0.0 : rest_32 < 0.35 ? 0.35 : rest_32));
       p->cfg = t_128 < t_32 ? 3 : 4;
       // Where the 128 x 128 ring tiles would sit one per CU (it is built for two, whose waves cover
       // each other's waits), the staged 64 x 256 tile - twice the row blocks per dequantised

@@ -206,6 +206,15 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
 
 
+def test_planner_keeps_small_batches_on_very_wide_layers_off_the_padded_tiles():
+    # a vocabulary-sized layer fills the 128 x 256 tiles' slots at any batch size; up to 64 batch rows
+    # those tiles would be mostly padding
+    assert _lib.describe_plan(4, 128, 128256, 4096, 32, True).endswith("cfg4")
+    assert _lib.describe_plan(4, 128, 128256, 4096, 17, True).endswith("cfg4")
+    assert _lib.describe_plan(4, 128, 128256, 4096, 128, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 128256, 4096, 2048, True).endswith("cfg0")
+
+
 def test_planner_takes_192_row_tiles_where_they_fill_one_round_better():
     # 6144 rows at M = 2048: 384 tiles of 128 x 256 leave half the CUs with one workgroup, 512 tiles
     # of 128 x 192 fill every slot; past 512 of them the wide tile is back
