@@ -369,6 +369,23 @@ def main() -> int:
                                         "moved_GBps": round(moved / t / 1e9, 1),
                                         "pct_hbm_peak_moved": round(moved / t / 1e9 / HBM_PEAK_GBPS * 100, 1),
                                         "presliced_us": table[f"{name}_b{b}_zp"]["us"]}
+            # batches of 8 and 64 rows at 4 bits from the same planes: the mid-batch kernel reads them
+            # itself (no workspace, no slicing pass); beside it the same kernel on the pre-sliced tensor
+            for m in (8, 64):
+                xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+                ym = torch.empty(m, n, dtype=torch.float16, device=dev)
+
+                def planes_call(i):
+                    _lib.check(L.matgptq_gemm_master(bits, GROUP, n, k, m, mring[i % cp].data_ptr(), aux[name][0].data_ptr(),
+                                                     aux[name][1].data_ptr(), xm.data_ptr(), ym.data_ptr(),
+                                                     None, 0, stream.cuda_stream, 1))
+                assert L.matgptq_gemm_master_workspace_bytes(bits, GROUP, n, k, m, 1) == 0
+                t = timed_graph(lambda: [planes_call(i) for i in range(cp)]) / cp
+                ring4 = rings[name]
+                tp = timed_graph(lambda: [launch(bits, n, k, xm, ring4[i % len(ring4)], aux[name][0], aux[name][1], ym)
+                                          for i in range(len(ring4))]) / len(ring4)
+                mtab[f"{name}_b{bits}_M{m}"] = {"us": round(t * 1e6, 2), "presliced_us": round(tp * 1e6, 2),
+                                                "moved_GBps": round(n * k * (bits + 1) / 8 / t / 1e9, 1)}
             del mring
         extra["gemv_M1_master_resident"] = mtab
         # ----------------------------------------- small batch (configs[2]), all four layers

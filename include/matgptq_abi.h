@@ -156,8 +156,9 @@ int matgptq_unpack_master_host(const uint32_t *planes_host, int64_t N, int64_t K
                                uint8_t *codes_host);
 int matgptq_unpack_master_device(const uint32_t *planes_dev, int64_t N, int64_t K, int bitwidth,
                                  uint8_t *codes_dev, void *stream);
-/* matgptq_gemm on master-resident planes.  Batch sizes 1..4 at group size 128 (the HBM-bound
- * regime, where the bytes moved decide) read the planes in the GEMM kernel itself.  Every other
+/* matgptq_gemm on master-resident planes.  Batch sizes 1..4 (the HBM-bound regime, where the
+ * bytes moved decide) and the mid-batch kernel - every shape up to 128 batch rows, and the larger
+ * batches that kernel is planned for anyway - read the planes in the GEMM kernel itself.  Every other
  * shape slices the planes into the pre-sliced layout first, in `workspace_dev`
  * (matgptq_gemm_master_workspace_bytes() bytes, 0 when none is needed), and runs the kernel of that
  * regime on it: two launches, no allocation.  Too small a workspace returns MATGPTQ_EWORKSPACE. */

@@ -24,10 +24,10 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
   hipError_t launch_decode_b##B(const GemmArgs&, int group_size, int R, int S, int W, int kc,  \
                                 bool stream_flavour, size_t smem, hipStream_t);                \
   hipError_t launch_prefill_b##B(const GemmArgs&, int group_size, int cfg, hipStream_t);          \
-  hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, hipStream_t);   \
+  hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, bool master, hipStream_t);   \
   hipError_t launch_gemv_b##B(const GemmArgs&, int group_size, int shape, int W, size_t lds_pad, bool master, hipStream_t);  \
   hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int group_size, int shape, int W, size_t lds_pad, bool master, hipStream_t); \
-  hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, hipStream_t); \
+  hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, bool master, hipStream_t); \
   hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
                                        int kc, bool stream_flavour, size_t smem, hipStream_t); \
   hipError_t launch_prefill_b##B##_bf16(const GemmArgs&, int group_size, int cfg, hipStream_t);
@@ -408,15 +408,15 @@ hipError_t launch_gemv(int bits, bool bf16, const GemmArgs& a, int g, const Plan
 #undef MATGPTQ_CASE
 }
 
-hipError_t launch_skinny(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, hipStream_t s) {
+hipError_t launch_skinny(int bits, bool bf16, const GemmArgs& a, int g, const Plan& p, bool master, hipStream_t s) {
 #define MATGPTQ_CASE(B) \
-  case B: return bf16 ? launch_skinny_b##B##_bf16(a, g, p.R, p.mb, s) : launch_skinny_b##B(a, g, p.R, p.mb, s);
+  case B: return bf16 ? launch_skinny_b##B##_bf16(a, g, p.R, p.mb, master, s) : launch_skinny_b##B(a, g, p.R, p.mb, master, s);
   switch (bits) {
     MATGPTQ_CASE(2)
     MATGPTQ_CASE(3)
     MATGPTQ_CASE(4)
     MATGPTQ_CASE(6)
-    default: return bf16 ? launch_skinny_b8_bf16(a, g, p.R, p.mb, s) : launch_skinny_b8(a, g, p.R, p.mb, s);
+    default: return bf16 ? launch_skinny_b8_bf16(a, g, p.R, p.mb, master, s) : launch_skinny_b8(a, g, p.R, p.mb, master, s);
   }
 #undef MATGPTQ_CASE
 }
@@ -451,8 +451,12 @@ const char* matgptq_strerror(int code) {
   }
 }
 
+// The kernels that read master-resident bit planes themselves: the gemv kernel in its two shapes
+// built for them, and the mid-batch kernel.
+static bool plan_reads_planes(const Plan& p) { return (p.gemv && (p.shape == 1 || p.shape == 2)) || p.skinny; }
+
 // checks, plan, launch; `master_planes`: the weight operand is master-resident bit planes and
-// the plan must be the gemv kernel (the caller has made sure of it)
+// the plan must be one of those kernels (the caller has made sure of it)
 static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M, const void* weights_dev,
                     const void* scales_dev, const void* zeros_dev, const void* x_dev, void* y_dev,
                     void* stream, uint32_t flags, bool master_planes) {
@@ -463,7 +467,7 @@ static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t 
   if (!weights_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &p)) return e;
-  if (master_planes && !(p.gemv && (p.shape == 1 || p.shape == 2))) return MATGPTQ_EVARIANT;
+  if (master_planes && !plan_reads_planes(p)) return MATGPTQ_EVARIANT;
   GemmArgs a;
   a.packed = static_cast<const uint32_t*>(weights_dev);
   a.scales = static_cast<const uint16_t*>(scales_dev);
@@ -480,7 +484,7 @@ static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t 
   const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
   const hipError_t err = p.gemv     ? launch_gemv(bitwidth, bf16, a, group_size, p, master_planes, s)
                          : p.decode ? launch_decode(bitwidth, bf16, a, group_size, p, s)
-                         : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, s)
+                         : p.skinny ? launch_skinny(bitwidth, bf16, a, group_size, p, master_planes, s)
                                     : launch_prefill(bitwidth, bf16, a, group_size, p, s);
   if (err != hipSuccess) return MATGPTQ_ELAUNCH;
   // K = 128 t + 64: the kernels above have multiplied the t tiles; a second launch adds the last 64 columns
@@ -498,23 +502,36 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
                   flags, false);
 }
 
-// does the GEMM at this shape read the planes itself (gemv kernel), or does it need the
-// pre-sliced tensor in a workspace first?
+// does the GEMM at this shape read the planes itself (gemv and mid-batch kernels), or does it need
+// the pre-sliced tensor in a workspace first?
+// `flags` comes back with the plan to take: up to 128 batch rows a shape whose own plan needs the
+// workspace is given the mid-batch kernel instead (its largest shape for that batch size), which
+// costs 1.05 .. 1.4 times its time on pre-sliced codes but saves the slicing pass - 41 us for the
+// 117 M codes of a 28672 x 4096 layer, more than such a product takes.
 static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M, bool zp,
-                               uint32_t flags, bool* direct) {
+                               uint32_t* flags, bool* direct) {
   if (int e = check_problem(bitwidth, group_size, N, K)) return e;
   if (K % 128 != 0) return MATGPTQ_ESHAPE;  // the bit planes have whole tiles only
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
-  if (int e = make_plan(bitwidth, group_size, N, K, M, zp, flags, &p)) return e;
-  *direct = p.gemv && (p.shape == 1 || p.shape == 2);
+  if (int e = make_plan(bitwidth, group_size, N, K, M, zp, *flags, &p)) return e;
+  *direct = plan_reads_planes(p);
+  const bool automatic = (*flags & MATGPTQ_FLAG_VARIANT_MASK) == 0 && ((*flags >> 16) & 3u) == 0;
+  if (!*direct && automatic && M > kGemvMaxM && M <= 128) {
+    const uint32_t msel = M <= 16 ? 0u : M <= 32 ? 1u : 2u;  // 16, 32 or 64 batch rows per workgroup
+    const uint32_t forced = *flags | ((80u + 2u + 3u * msel) << MATGPTQ_FLAG_VARIANT_SHIFT);  // four row blocks, or as many as fit
+    if (make_plan(bitwidth, group_size, N, K, M, zp, forced, &p) == MATGPTQ_OK && plan_reads_planes(p)) {
+      *flags = forced;
+      *direct = true;
+    }
+  }
   return MATGPTQ_OK;
 }
 
 size_t matgptq_gemm_master_workspace_bytes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
                                            uint32_t flags) {
   bool direct = false;
-  if (master_reads_planes(bitwidth, group_size, N, K, M, true, flags, &direct) != MATGPTQ_OK) return 0;
+  if (master_reads_planes(bitwidth, group_size, N, K, M, true, &flags, &direct) != MATGPTQ_OK) return 0;
   return direct ? 0 : matgptq_packed_words(bitwidth, N, K) * 4;
 }
 
@@ -523,7 +540,7 @@ static int gemm_master_impl(int bitwidth, int group_size, int64_t N, int64_t K, 
                             const void* x_dev, void* y_dev, void* workspace_dev, size_t workspace_bytes,
                             void* stream, uint32_t flags) {
   bool direct = false;
-  if (int e = master_reads_planes(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &direct)) return e;
+  if (int e = master_reads_planes(bitwidth, group_size, N, K, M, zeros_dev != nullptr, &flags, &direct)) return e;
   if (!planes_dev) return MATGPTQ_ENULL;
   if (direct)
     return run_gemm(bitwidth, group_size, N, K, M, planes_dev, scales_dev, zeros_dev, x_dev, y_dev, stream,
@@ -568,7 +585,8 @@ int matgptq_gemm_master_static(int bitwidth, int group_size, int64_t N, int64_t 
                                const void* planes_dev, const void* scales_dev, const void* zeros_dev,
                                const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
   bool direct = false;
-  if (int e = master_reads_planes(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &direct)) return e;
+  uint32_t plan_flags = flags;  // (gemm_master_impl decides again from the caller's flags, the same way)
+  if (int e = master_reads_planes(bitwidth, group_size, N, K, M, zeros_dev != nullptr, &plan_flags, &direct)) return e;
   void* ws = nullptr;
   size_t need = 0;
   if (!direct) {

@@ -35,7 +35,7 @@
 //
 // The activations are re-read once per workgroup column (N / (16 R) times in total, from L2):
 // that traffic, not the weights, bounds this kernel, which is why R grows with N.
-#include "device_common.h"
+#include "tile_format.h"
 
 #ifndef MATGPTQ_BITS
 #error "compile with -DMATGPTQ_BITS={2,3,4,6,8}"
@@ -56,9 +56,12 @@ constexpr int skinny_lds_bytes(int r, int mb) {
   return stage > sums ? stage : sums;
 }
 
-template <int BITS, int GROUP, bool ZP, int R, int MB>
+// MASTER: `a.packed` holds the master-resident bit planes (master_layout.h); the slice to BITS,
+// rounding and saturation happen in registers on the way to the raw fp16 pairs.
+template <int BITS, int GROUP, bool ZP, int R, int MB, bool MASTER>
 __global__ void __launch_bounds__(64 * kWaves, 2)
 skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
+  using Fmt = TileFormat<BITS, MASTER>;
   constexpr int GPT = GROUP == 32 ? 4 : 1;
   constexpr int kStage = MB * 16 * 256;  // bytes of one activation buffer
   constexpr int NS = 2;  // register sets of codes, scales, zeros
@@ -79,7 +82,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   const int m0 = (lid - nt * m_tiles) * (16 * MB);
   const int rb_first = nt * R;
 
-  constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
+  constexpr uint32_t tile_bytes = Fmt::kTileBytes;
   const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
   const uint32_t w_bytes = (uint32_t)a.row_blocks * rb_bytes;
   const uint32_t aux_bytes = (uint32_t)a.row_blocks * a.G * 32;  // scales / zeros: [N/16][G][16] halves
@@ -91,13 +94,13 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
 #pragma unroll
     for (int i = 0; i < MB; i++) acc[rr][i] = float4v{0.f, 0.f, 0.f, 0.f};
 
-  const UnpackConsts<BITS> kc_unpack;
+  const typename Fmt::Consts kc_unpack;
   const float kc_zero = __uint_as_float(opaque_vgpr(0u));  // a zero the optimiser cannot see through
   // codes, scales and zeros of the tile in use and of the next one; scales and zeros stay as
   // loaded and are converted where they are used
-  uint32_t wr[NS][R][BITS], sr[NS][R][GPT], zr[NS][R][GPT];
+  uint32_t wr[NS][R][Fmt::kWords], sr[NS][R][GPT], zr[NS][R][GPT];
 
-  auto load_weights = [&](uint32_t (&w)[R][BITS], uint32_t (&s)[R][GPT], uint32_t (&z)[R][GPT], int kb) {
+  auto load_weights = [&](uint32_t (&w)[R][Fmt::kWords], uint32_t (&s)[R][GPT], uint32_t (&z)[R][GPT], int kb) {
 #pragma unroll
     for (int rr = 0; rr < R; rr++) {
       const int rb = rb_first + rr;
@@ -105,7 +108,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
       const BufRsrc wr = make_rsrc(a.packed, valid ? w_bytes : 0u);
       const BufRsrc sr = make_rsrc(a.scales, valid ? aux_bytes : 0u);
       const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, valid ? aux_bytes : 0u);
-      load_tile_words<BITS, 0>(wr, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
+      Fmt::template load<0>(wr, (uint32_t)rb * rb_bytes + (uint32_t)kb * tile_bytes, lane, w[rr]);
 #pragma unroll
       for (int gg = 0; gg < GPT; gg++) {
         const uint32_t g = GROUP == -1 ? 0u : (uint32_t)kb * GPT + gg;
@@ -143,7 +146,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
     return *reinterpret_cast<const half8*>(stage + (i * 16 + r16) * 256 + (((4 * j + q) ^ r16) * 16));
   };
 
-  auto dequant_step = [&](Frag (&aw)[R], const uint32_t (&w)[R][BITS], const uint32_t (&s)[R][GPT],
+  auto dequant_step = [&](Frag (&aw)[R], const uint32_t (&w)[R][Fmt::kWords], const uint32_t (&s)[R][GPT],
                           const uint32_t (&z)[R][GPT], auto jtag) {
     constexpr int J = decltype(jtag)::value;
 #pragma unroll
@@ -156,7 +159,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
         const float sm = s0 * (float)(1 << (8 - BITS));
         float sz = kc_zero;
         if constexpr (ZP) sz = s0 * (bf16_bits_to_float(z[rr][gg]) - 128.0f);
-        dequant_octet_bf16<BITS, J>(w[rr], kc_unpack, sm, sz, aw[rr]);
+        dequant_octet_bf16_fmt<Fmt, BITS, J>(w[rr], kc_unpack, sm, sz, aw[rr]);
       } else {
         // fp16 storage: scale * 2^(8-b) and scale * (zero - 128)
         const _Float16 s0 = __builtin_bit_cast(_Float16, (uint16_t)s[rr][gg]);
@@ -165,7 +168,7 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
         if constexpr (ZP) z1 = s0 * (__builtin_bit_cast(_Float16, (uint16_t)z[rr][gg]) - (_Float16)128.0f);
         const half2v sc = {s1, s1};
         const half2v zr = {z1, z1};
-        dequant_octet<BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
+        dequant_octet_fmt<Fmt, BITS, J, ZP>(w[rr], kc_unpack, zr, sc, aw[rr]);
       }
     }
   };
@@ -253,30 +256,36 @@ skinny_kernel(const GemmArgs a, int n_tiles, int m_tiles) {
   }
 }
 
-template <int GROUP, bool ZP, int R, int MB>
+template <int GROUP, bool ZP, int R, int MB, bool MASTER>
 hipError_t launch_r(const GemmArgs& a, hipStream_t stream) {
   const int n_tiles = (a.row_blocks + R - 1) / R;
   const int m_tiles = (a.M + 16 * MB - 1) / (16 * MB);
   const dim3 grid(n_tiles * m_tiles), block(64 * kWaves);
-  hipLaunchKernelGGL((skinny_kernel<kBits, GROUP, ZP, R, MB>), grid, block, 0, stream, a, n_tiles, m_tiles);
+  hipLaunchKernelGGL((skinny_kernel<kBits, GROUP, ZP, R, MB, MASTER>), grid, block, 0, stream, a, n_tiles, m_tiles);
   return hipGetLastError();
 }
 
-template <int GROUP, bool ZP, int MB>
+template <int GROUP, bool ZP, int MB, bool MASTER>
 hipError_t launch_rows(const GemmArgs& a, int r, hipStream_t s) {
   // (four row blocks fit the register budget of two waves per SIMD up to 6 bits and with one
-  // scale and zero per tile and row block; group 32 carries four)
-  if constexpr (GROUP != 32 && kBits <= 6) {
-    if (r >= 4) return launch_r<GROUP, ZP, 4, MB>(a, s);
+  // scale and zero per tile and row block; group 32 carries four; the master planes are eight
+  // words per lane from 6 bits on)
+  if constexpr (GROUP != 32 && kBits <= (MASTER ? 4 : 6)) {
+    if (r >= 4) return launch_r<GROUP, ZP, 4, MB, MASTER>(a, s);
   }
-  if (r >= 2) return launch_r<GROUP, ZP, 2, MB>(a, s);
-  return launch_r<GROUP, ZP, 1, MB>(a, s);
+  if (r >= 2) return launch_r<GROUP, ZP, 2, MB, MASTER>(a, s);
+  return launch_r<GROUP, ZP, 1, MB, MASTER>(a, s);
+}
+
+template <int GROUP, bool ZP, bool MASTER>
+hipError_t launch_batch(const GemmArgs& a, int r, int mb, hipStream_t s) {
+  if (mb >= 4) return launch_rows<GROUP, ZP, 4, MASTER>(a, r, s);
+  return mb >= 2 ? launch_rows<GROUP, ZP, 2, MASTER>(a, r, s) : launch_rows<GROUP, ZP, 1, MASTER>(a, r, s);
 }
 
 template <int GROUP, bool ZP>
-hipError_t launch_batch(const GemmArgs& a, int r, int mb, hipStream_t s) {
-  if (mb >= 4) return launch_rows<GROUP, ZP, 4>(a, r, s);
-  return mb >= 2 ? launch_rows<GROUP, ZP, 2>(a, r, s) : launch_rows<GROUP, ZP, 1>(a, r, s);
+hipError_t launch_storage(const GemmArgs& a, int r, int mb, bool master, hipStream_t s) {
+  return master ? launch_batch<GROUP, ZP, true>(a, r, mb, s) : launch_batch<GROUP, ZP, false>(a, r, mb, s);
 }
 
 }  // namespace
@@ -289,13 +298,14 @@ hipError_t launch_batch(const GemmArgs& a, int r, int mb, hipStream_t s) {
 #else
 #define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_skinny_b, MATGPTQ_BITS)
 #endif
-hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int r, int mb, hipStream_t stream) {
+// master: `a.packed` holds master-resident bit planes
+hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int r, int mb, bool master, hipStream_t stream) {
   const bool zp = a.zeros != nullptr;
   if (group_size == 128)
-    return zp ? launch_batch<128, true>(a, r, mb, stream) : launch_batch<128, false>(a, r, mb, stream);
+    return zp ? launch_storage<128, true>(a, r, mb, master, stream) : launch_storage<128, false>(a, r, mb, master, stream);
   if (group_size == 32)
-    return zp ? launch_batch<32, true>(a, r, mb, stream) : launch_batch<32, false>(a, r, mb, stream);
-  return zp ? launch_batch<-1, true>(a, r, mb, stream) : launch_batch<-1, false>(a, r, mb, stream);
+    return zp ? launch_storage<32, true>(a, r, mb, master, stream) : launch_storage<32, false>(a, r, mb, master, stream);
+  return zp ? launch_storage<-1, true>(a, r, mb, master, stream) : launch_storage<-1, false>(a, r, mb, master, stream);
 }
 
 }  // namespace matgptq

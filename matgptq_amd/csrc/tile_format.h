@@ -18,8 +18,10 @@ struct TileFormat<BITS, false> {
   static constexpr bool kScaledX = BITS != 8;  // some pair has p != 0
   static constexpr int raw_shift(int j, int i) { return Codec<BITS>::raw_shift(j, i); }
   using Consts = UnpackConsts<BITS>;
+  // AUX: the cache policy of the loads (kAuxStream for data read once, 0 for data other workgroups read again)
+  template <int AUX = kAuxStream>
   __device__ __forceinline__ static void load(BufRsrc rs, uint32_t tile_off, int lane, uint32_t (&w)[kWords]) {
-    load_tile_words<BITS>(rs, tile_off, lane, w);
+    load_tile_words<BITS, AUX>(rs, tile_off, lane, w);
   }
   template <int J>
   __device__ __forceinline__ static void raw(const uint32_t (&w)[kWords], const Consts& k, uint32_t (&r)[4]) {
@@ -37,13 +39,14 @@ struct TileFormat<BITS, true> {
   static constexpr int raw_shift(int /*j*/, int i) { return BITS <= 4 ? ((i & 1) ? 4 : 0) : 0; }
   using Consts = UnpackConsts<4>;  // nibble masks and the magic word
   // one load per segment the bitwidth reads (S0: 12 bytes per lane, S1, S2: 4, S3: 12)
+  template <int AUX = kAuxStream>
   __device__ __forceinline__ static void load(BufRsrc rs, uint32_t tile_off, int lane, uint32_t (&w)[kWords]) {
-    const u32x3 a = __builtin_amdgcn_raw_buffer_load_b96(rs, lane * 12, tile_off, kAuxStream);
+    const u32x3 a = __builtin_amdgcn_raw_buffer_load_b96(rs, lane * 12, tile_off, AUX);
     w[0] = a.x; w[1] = a.y; w[2] = a.z;
-    if constexpr (BITS >= 3) w[3] = __builtin_amdgcn_raw_buffer_load_b32(rs, 768 + lane * 4, tile_off, kAuxStream);
-    if constexpr (BITS >= 4) w[4] = __builtin_amdgcn_raw_buffer_load_b32(rs, 1024 + lane * 4, tile_off, kAuxStream);
+    if constexpr (BITS >= 3) w[3] = __builtin_amdgcn_raw_buffer_load_b32(rs, 768 + lane * 4, tile_off, AUX);
+    if constexpr (BITS >= 4) w[4] = __builtin_amdgcn_raw_buffer_load_b32(rs, 1024 + lane * 4, tile_off, AUX);
     if constexpr (BITS >= 6) {
-      const u32x3 c = __builtin_amdgcn_raw_buffer_load_b96(rs, 1280 + lane * 12, tile_off, kAuxStream);
+      const u32x3 c = __builtin_amdgcn_raw_buffer_load_b96(rs, 1280 + lane * 12, tile_off, AUX);
       w[5] = c.x; w[6] = c.y; w[7] = c.z;
     }
   }
@@ -67,6 +70,29 @@ struct TileFormat<BITS, true> {
     }
   }
 };
+
+// Octet J of a tile in either storage -> the 16 x 32 MFMA operand of dequantised weights (the
+// arithmetic of dequant_octet / dequant_octet_bf16 in device_common.h on the format's raw pairs).
+template <class Fmt, int BITS, int J, bool ZP>
+__device__ __forceinline__ void dequant_octet_fmt(const uint32_t (&w)[Fmt::kWords], const typename Fmt::Consts& k,
+                                                  half2v zrel, half2v scale, Frag& a) {
+  uint32_t raw[4];
+  Fmt::template raw<J>(w, k, raw);
+  a.p[0] = dequant_pair<BITS, Fmt::raw_shift(J, 0), ZP>(raw[0], zrel, scale);
+  a.p[1] = dequant_pair<BITS, Fmt::raw_shift(J, 1), ZP>(raw[1], zrel, scale);
+  a.p[2] = dequant_pair<BITS, Fmt::raw_shift(J, 2), ZP>(raw[2], zrel, scale);
+  a.p[3] = dequant_pair<BITS, Fmt::raw_shift(J, 3), ZP>(raw[3], zrel, scale);
+}
+template <class Fmt, int BITS, int J>
+__device__ __forceinline__ void dequant_octet_bf16_fmt(const uint32_t (&w)[Fmt::kWords], const typename Fmt::Consts& k,
+                                                       float sm, float sz, Frag& a) {
+  uint32_t raw[4];
+  Fmt::template raw<J>(w, k, raw);
+  a.u[0] = dequant_pair_bf16<BITS, Fmt::raw_shift(J, 0)>(raw[0], sm, sz);
+  a.u[1] = dequant_pair_bf16<BITS, Fmt::raw_shift(J, 1)>(raw[1], sm, sz);
+  a.u[2] = dequant_pair_bf16<BITS, Fmt::raw_shift(J, 2)>(raw[2], sm, sz);
+  a.u[3] = dequant_pair_bf16<BITS, Fmt::raw_shift(J, 3)>(raw[3], sm, sz);
+}
 
 // Number of load instructions TileFormat::load issues for one tile.
 constexpr int master_load_count(int bits) { return bits == 2 ? 1 : bits == 3 ? 2 : bits == 4 ? 3 : 4; }

@@ -91,16 +91,72 @@ def test_exact_in_the_reference_test_regime():
             assert np.array_equal(y.view(np.uint16), o.linear_f64(x, w).astype(np.float16).view(np.uint16)), (b, m)
 
 
-@pytest.mark.parametrize("b,g,m", [(4, 128, 8), (3, 128, 16), (4, 128, 64), (6, 128, 300), (2, 32, 5), (8, -1, 13), (4, 32, 40)])
-def test_shapes_outside_the_gemv_kernel_go_through_the_workspace(b, g, m):
+@pytest.mark.parametrize("b,g,m", [(4, 128, 8), (3, 128, 16), (4, 128, 64), (6, 128, 300), (2, 32, 5), (8, -1, 13), (4, 32, 40),
+                                   (2, 128, 100), (8, 32, 33), (6, -1, 7), (3, 32, 513), (6, 128, 1000)])
+def test_midbatch_kernel_reads_the_planes_itself(b, g, m):
     n, k = 304, 1024
     q, s, z = o.make_layer(n, k, g, seed=b + m)
     planes = planes_device(q)
     sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
     x = o.make_activations(m, k, seed=m)
+    assert _lib.describe_plan(b, g, n, k, m, True).startswith("midbatch")
+    for zeros in (zr, None):
+        y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zeros, workspace=None)
+        assert need == 0
+        zz = z if zeros is not None else np.full_like(z, 128)
+        G.assert_close_to_oracle(y, x, o.dequantize(q, s, zz, b, g), f"planes, mid-batch b={b} g={g} M={m}")
+        # bit-identical to the pre-sliced tensor: the same codes reach the same arithmetic
+        y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zeros).cpu().numpy()
+        assert np.array_equal(y, y2)
+
+
+@pytest.mark.parametrize("r,mb", [(1, 1), (2, 1), (4, 1), (1, 2), (2, 2), (4, 2), (1, 4), (2, 4), (4, 4)])
+def test_midbatch_kernel_from_planes_every_shape(r, mb):
+    # every (row blocks, batch rows) shape of the kernel forced, on codes that hit the rounding
+    # carry and the saturation of the slice (all 256 master values occur)
+    n, k, m = 208, 128 * 9, 70
+    rng = np.random.default_rng(r * 10 + mb)
+    q = rng.integers(0, 256, (n, k), dtype=np.uint8)
+    q[0, :256] = np.arange(256, dtype=np.uint8)
+    _, s, z = o.make_layer(n, k, 128, seed=3)
+    planes = planes_device(q)
+    sc, zr = G.reorder_device(s, n, k, 128), G.reorder_device(z, n, k, 128)
+    x = o.make_activations(m, k, seed=4)
+    flags = 1 | ((80 + {1: 0, 2: 1, 4: 2}[r] + 3 * {1: 0, 2: 1, 4: 2}[mb]) << 8)
+    for b in BITS:
+        y, need = gemm_master(b, 128, n, k, G.to_dev(x), planes, sc, zr, flags=flags, workspace=None)
+        assert need == 0
+        G.assert_close_to_oracle(y, x, o.dequantize(q, s, z, b, 128), f"planes, mid-batch R{r} mb{mb} b={b}")
+        y2 = G.gemm(b, 128, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zr, flags).cpu().numpy()
+        assert np.array_equal(y, y2)
+
+
+@pytest.mark.parametrize("b,m", [(8, 8), (8, 16), (4, 128), (6, 100), (2, 64)])
+def test_many_row_layers_take_the_midbatch_kernel_on_planes(b, m):
+    # the plan for the pre-sliced tensor is another kernel here (decode or a prefill tile); on planes the
+    # mid-batch kernel saves the slicing pass up to 128 batch rows
+    n, k, g = 16384 + 16, 1024, 128
+    q, s, z = o.make_layer(n, k, g, seed=b * m)
+    planes = planes_device(q)
+    sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
+    x = o.make_activations(m, k, seed=m)
+    y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zr, workspace=None)
+    assert need == 0
+    G.assert_close_to_oracle(y, x, o.dequantize(q, s, z, b, g), f"planes, many rows b={b} M={m}")
+    G.assert_regression_bound(y, x, o.dequantize(q, s, z, b, g), f"planes, many rows b={b} M={m}")
+
+
+@pytest.mark.parametrize("b,g,n,k,m", [(8, 128, 304, 1024, 2048), (4, 128, 2048, 1024, 700), (6, 32, 1024, 512, 1500)])
+def test_shapes_outside_those_kernels_go_through_the_workspace(b, g, n, k, m):
+    q, s, z = o.make_layer(n, k, g, seed=b + m)
+    planes = planes_device(q)
+    sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
+    x = o.make_activations(m, k, seed=m)
+    assert _lib.describe_plan(b, g, n, k, m, True).startswith("prefill")
     y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zr)
     assert need == b * n * k // 8
-    G.assert_close_to_oracle(y, x, o.dequantize(q, s, z, b, g), f"workspace path b={b} g={g} M={m}")
+    rows = np.r_[0:16, m - 16:m]
+    G.assert_close_to_oracle(y[rows], x[rows], o.dequantize(q, s, z, b, g), f"workspace path b={b} g={g} M={m}")
     # bit-identical to the pre-sliced tensor: the second launch is the same kernel on the same codes
     y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zr).cpu().numpy()
     assert np.array_equal(y, y2)

@@ -107,13 +107,20 @@ def test_error_codes():
     assert lib.matgptq_pack_master_host(1, 15, 128, 1) == -3
     assert lib.matgptq_unpack_master_host(1, 16, 128, 5, 1) == -1
     assert lib.matgptq_gemm_master(4, 128, 16, 128, 1, None, 1, None, 1, 1, None, 0, None, 1) == -4
-    # outside the batch-1..4 kernel a workspace is needed
+    # the batch-1..4 kernel and the mid-batch kernel read the planes themselves; outside them a
+    # workspace is needed
     assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 4096, 4096, 1, 1) == 0
     assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 4096, 4096, 4, 1) == 0
-    assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 4096, 4096, 5, 1) == 4096 * 4096 // 2
+    assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 4096, 4096, 5, 1) == 0
     assert lib.matgptq_gemm_master_workspace_bytes(3, 32, 4096, 4096, 1, 1) == 0
-    assert lib.matgptq_gemm_master_workspace_bytes(3, 32, 4096, 4096, 7, 1) == 3 * 4096 * 4096 // 8
+    assert lib.matgptq_gemm_master_workspace_bytes(3, 32, 4096, 4096, 7, 1) == 0
+    assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 4096, 4096, 64, 1) == 0
+    # (up to 128 batch rows a shape whose own plan is another kernel takes the mid-batch kernel here)
+    assert lib.matgptq_gemm_master_workspace_bytes(8, 128, 28672, 4096, 8, 1) == 0
+    assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 28672, 4096, 128, 1) == 0
+    assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 28672, 4096, 129, 1) == 28672 * 4096 // 2
+    assert lib.matgptq_gemm_master_workspace_bytes(8, 128, 28672, 4096, 8, 1 | (1 << 16)) == 28672 * 4096   # decode kernel asked for
     assert lib.matgptq_gemm_master_workspace_bytes(4, 128, 4096, 4096, 2048, 1) == 4096 * 4096 // 2
-    assert lib.matgptq_gemm_master(4, 128, 4096, 4096, 64, 1, 1, None, 1, 1, None, 0, None, 1) == -9
-    assert lib.matgptq_gemm_master(4, 128, 4096, 4096, 64, 1, 1, None, 1, 1, 1, 100, None, 1) == -9
+    assert lib.matgptq_gemm_master(4, 128, 4096, 4096, 2048, 1, 1, None, 1, 1, None, 0, None, 1) == -9
+    assert lib.matgptq_gemm_master(4, 128, 4096, 4096, 2048, 1, 1, None, 1, 1, 1, 100, None, 1) == -9
     assert "workspace" in lib.matgptq_strerror(-9).decode()
