@@ -463,7 +463,8 @@ def main() -> int:
                         launch(4, n, k, xm, packed, sc, zr, ym)
                     stream.synchronize()
             for zp in (True, False):
-                t = timed_graph(lambda: [launch(4, n, k, xm, packed, sc, zr if zp else None, ym) for _ in range(5)]) / 5
+                t = timed_graph(lambda: [launch(4, n, k, xm, packed, sc, zr if zp else None, ym) for _ in range(5)],
+                                settle_ms=20.0) / 5
                 tf = 2.0 * m * n * k / t / 1e12
                 pre[f"{name}_b4_M2048_{'zp' if zp else 'sym'}"] = {
                     "ms": round(t * 1e3, 3), "TFLOPs": round(tf, 1),
@@ -471,7 +472,7 @@ def main() -> int:
             # the other bitwidths (zero-point form) and bf16 storage at 4 bits
             for b in (2, 3, 6, 8):
                 pk = make_ring(n, k, b, 1)[0]
-                t = timed_graph(lambda: [launch(b, n, k, xm, pk, sc, zr, ym) for _ in range(3)], reps=3) / 3
+                t = timed_graph(lambda: [launch(b, n, k, xm, pk, sc, zr, ym) for _ in range(3)], reps=3, settle_ms=20.0) / 3
                 tf = 2.0 * m * n * k / t / 1e12
                 pre[f"{name}_b{b}_M2048_zp"] = {"ms": round(t * 1e3, 3), "TFLOPs": round(tf, 1),
                                                 "pct_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS * 100, 1),
@@ -479,7 +480,8 @@ def main() -> int:
                 del pk
             xb, scb, zrb = xm.to(torch.bfloat16), sc.to(torch.bfloat16), zr.to(torch.bfloat16)
             yb = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
-            t = timed_graph(lambda: [launch(4, n, k, xb, packed, scb, zrb, yb, flags=3) for _ in range(3)], reps=3) / 3
+            t = timed_graph(lambda: [launch(4, n, k, xb, packed, scb, zrb, yb, flags=3) for _ in range(3)], reps=3,
+                            settle_ms=20.0) / 3
             tf = 2.0 * m * n * k / t / 1e12
             pre[f"{name}_b4_M2048_zp_bf16"] = {"ms": round(t * 1e3, 3), "TFLOPs": round(tf, 1),
                                                "pct_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS * 100, 1),
