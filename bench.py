@@ -125,11 +125,12 @@ def main() -> int:
         zeros = torch.randint(0, 256, (groups,), device=dev, generator=g).to(torch.float16)
         return scales, zeros
 
-    def timed_graph(build, reps=5, settle_ms=0.0):
+    def timed_graph(build, reps=5, settle_ms=10.0):
         """Captures `build()` (launches on `stream`) into a HIP graph; returns the median
         replay time in seconds over `reps` replays, measured with events on `stream`.
         `settle_ms`: keep replaying, untimed, for that long first (the clocks take some
-        milliseconds to settle after the allocation and random fill of a new ring of weights)."""
+        milliseconds to settle after the allocation and random fill of new tensors: a boost, then
+        a dip below the sustained clock; rows timed inside it read up to 20 % off either way)."""
         with torch.cuda.stream(stream):
             build()  # eager warm-up of every kernel in the graph
             stream.synchronize()
@@ -241,7 +242,7 @@ def main() -> int:
         stream.synchronize()
     torch.cuda.synchronize()
     t_wall0 = time.perf_counter()
-    elapsed = timed_graph(lambda: [step(i) for i in range(args.steps)], reps=21)  # median of 21 replays
+    elapsed = timed_graph(lambda: [step(i) for i in range(args.steps)], reps=21, settle_ms=0.0)  # median of 21 replays
     torch.cuda.synchronize()
     t_wall = time.perf_counter() - t_wall0
     ms_per_step = elapsed / args.steps * 1e3
@@ -253,7 +254,7 @@ def main() -> int:
     t_dom = timed_graph(lambda: [launch(bits, n, k, x_ring["gate_up"][i % copies], rings["gate_up"][i % copies],
                                         aux_ring["gate_up"][i % copies][0], aux_ring["gate_up"][i % copies][1],
                                         ys["gate_up"])
-                                 for i in range(launches)], reps=21) / launches
+                                 for i in range(launches)], reps=21, settle_ms=0.0) / launches
     dom_bytes = algorithmic_bytes(n, k, 1, bits)
     roofline = {
         "kernel": _lib.describe_plan(bits, GROUP, n, k, 1, True),
@@ -313,7 +314,7 @@ def main() -> int:
                 for zp in (True, False):
                     t = timed_graph(lambda: [launch(b, n, k, xs[name], ring[i % cp], aux[name][0],
                                                     aux[name][1] if zp else None, ys[name])
-                                             for i in range(reps)], settle_ms=0.0 if b == bits else 15.0) / reps
+                                             for i in range(reps)], settle_ms=15.0) / reps
                     table[f"{name}_b{b}_{'zp' if zp else 'sym'}"] = {
                         "us": round(t * 1e6, 2),
                         "weight_GBps": round(wbytes / t / 1e9, 1),
