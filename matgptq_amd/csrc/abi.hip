@@ -159,9 +159,14 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // resident workgroups as well (57344 x 8192, 6 bits: 1748 against 1906 us; on 8192 rows, 43
       // tiles of 192, it only ties).  Rounds times tile width decide.
       // bf16 storage dequantises through fp32 for the bf16 matrix instruction (four vector
-      // instructions per pair of weights instead of two): the wider tiles spill or stall on that
-      // work, the 128 x 128 tile does not, and except at 6 bits neither does the 128 x 192 tile
-      // (Llama-3-70B gate_up, M = 2048, 4 bits: 1590 against 1768 us; the 128 x 256 tile takes 2241).
+      // instructions per pair of weights instead of three).  At 2 and 4 bits, and at 8 bits with one
+      // scale per row, the 128 x 256 tile holds that in registers and the rules of fp16 storage apply
+      // (M = 2048, 4 bits: 8192 x 8192 228 against 256 us on 128 x 128 tiles, 8192 x 28672 761 against 870,
+      // 57344 x 8192 1542 against 1611 on 128 x 192).  At 3 and 6 bits, with group size 32, and at 8 bits
+      // with a scale and zero per tile it spills (8 bits, 8192 x 8192: 511 us): those take the
+      // 128 x 128 tile or, except at 6 bits, the 128 x 192 tile where its rounds pay.  8-bit codes fit
+      // the 128 x 256 tile again once eight waves halve K between them, up to two rounds of one such
+      // workgroup per CU (8192 x 8192, M = 2048: 243 against 270 us; 8192 x 28672: 889 against 1018).
       // Group size 32 with zero points keeps four scales and four zeros per tile and row block in
       // two register sets: the 128 x 256 tile spills (8192 x 8192, M = 2048: 489 us at 4 bits, 3023 us
       // at 8 bits, against 290 and 307 us on the 128 x 128 tile); the 128 x 192 tile fits up to 4 bits
@@ -170,10 +175,15 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       const bool g32zp = group_size == 32 && zp;
       const int64_t wgs_192 = ((N + 191) / 192) * m_tiles, wgs_128 = ((N + 127) / 128) * m_tiles;
       const bool fits_192 = !(bf16 && (bits == 6 || group_size == 32)) && !(bits == 6 && g32zp);
-      if (bits == 6 || bf16 || g32zp) {
-        const double t_192 = (double)((wgs_192 + 511) / 512) * 1.5 / 1.09;
-        const double t_128 = (double)((wgs_128 + 511) / 512);
+      const bool bf16_narrow =
+          bf16 && (group_size == 32 || !(bits == 2 || bits == 4 || (bits == 8 && group_size == -1)));
+      if (bits == 6 || bf16_narrow || g32zp) {
+        // (whole rounds of 512 resident workgroups up to two; beyond, the rounds blur into each other)
+        auto rounds = [](int64_t w) { return w <= 1024 ? (double)((w + 511) / 512) : (double)w / 512.0 + 0.5; };
+        const double t_192 = rounds(wgs_192) * 1.5 / 1.09;
+        const double t_128 = rounds(wgs_128);
         p->cfg = t_192 < t_128 && fits_192 ? 9 : 3;
+        if (p->cfg == 3 && bf16 && bits == 8 && group_size != 32 && wgs_big <= 512) p->cfg = 11;
       } else if (wgs_192 <= 512 && fits_192) {
         // Fewer than 512 of the 128 x 256 tiles leave half of the CUs with one workgroup where the
         // kernel is built for two; 128 x 192 tiles that still fit one round of 512 spread the same
@@ -212,12 +222,13 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // 64 x 256 tile, 8192 x 28672 249 against 298; 4096 x 4096 at M = 1024 40 against 48); 128 x 256 where
       // only these number at most the CUs, 5 us + 1.4 .. 1.65 per K tile (8192 x 8192 at M = 1024 111
       // against 125 us on 128 x 128 tiles two per CU, 8192 x 28672 366 against 440), for the formats
-      // whose registers fit that tile.
+      // whose registers fit that tile (bf16 storage: all but 3 and 6 bits and group size 32 -
+      // 8192 x 8192 at M = 1024 116 against 128 us at 4 bits, 127 against 148 at 8).
       const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
       if (wgs_128 <= 256) {
         const double t = 3.0 + kt * (1.0 + 0.12 * (double)wgs_128 / 256.0);
         if (t < best) { best = t; p->cfg = 10; }
-      } else if (wgs_big <= 256 && bits != 6 && !bf16 && !(group_size == 32 && zp)) {
+      } else if (wgs_big <= 256 && bits != 6 && !(bf16 && (bits == 3 || group_size == 32)) && !(group_size == 32 && zp)) {
         const double t = 5.0 + kt * (wgs_big > 192 ? 1.65 : 1.4);
         if (t < best) { best = t; p->cfg = 11; }
       }
@@ -227,11 +238,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         const int64_t wgs = (int64_t)((row_blocks + r - 1) / r) * m_tiles;
         // One workgroup per CU and round.  (With 32 batch rows and at most two row blocks a second
         // one fits, but two together take 1.6 times as long as one: 0.8 of the cost per tile each.)
-        // 8-bit codes cost 1.1 times as much per tile, bf16 storage (weights formed in fp32) 1.12
-        // times: 8192 x 8192, M = 256, 64 batch rows per workgroup: 49.5 us fp16, 53.8 us bf16.
+        // 8-bit codes cost 1.1 times as much per tile, bf16 storage (weights formed in fp32) 1.05
+        // times.
         const int64_t slots = 256;
         const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (mb == 2 && r <= 2 ? 0.8 : 1.0) *
-                                (bits == 8 ? 1.1 : 1.0) * (bf16 ? 1.12 : 1.0);
+                                (bits == 8 ? 1.1 : 1.0) * (bf16 ? 1.05 : 1.0);
         const int64_t rounds = (wgs + slots - 1) / slots;
         // (More than a thousand batch rows in more than one round: every XCD then streams most of
         // the activations through its 4 MB of L2 once per round, and the small staged tile is ahead -

@@ -263,13 +263,28 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float float2v __attribute__((ext_vector_type(2)));
 
+// The centring of the raw pair rides in the same fused multiply-add: with r = 1024 + c 2^P,
+//   scale (m c - zero) = r (sm 2^-P) - (sz + (1024 2^-P + centre) sm),
+// both constants per (row, group, P), formed once and exact in fp32 as long as the integer
+// 255 (128 + m (1024 2^-P + centre)) stays below 2^24 (every pair but the P = 0 pairs of 2-bit codes,
+// which keep the separate centring step).
 template <int BITS, int P>
 __device__ __forceinline__ uint32_t dequant_pair_bf16(uint32_t raw, float sm, float sz) {
-  const half2v u = centre_raw<P>(raw, Codec<BITS>::kCentre);
+  constexpr int kM = 1 << (8 - BITS);
+  constexpr bool kFold = 255ll * (128 + (long long)kM * ((1024 >> P) + Codec<BITS>::kCentre)) < (1ll << 24) && (1024 >> P) << P == 1024;
   // (symmetric layers pass an opaque zero as `sz`: the fused form is one instruction per element,
   // a conversion followed by a multiplication two)
-  const float2v w = {__builtin_fmaf((float)u.x, sm, -sz), __builtin_fmaf((float)u.y, sm, -sz)};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));
+  if constexpr (kFold) {
+    const half2v r = h2_from_bits(raw);
+    const float sp = sm * (1.0f / (float)(1 << P));
+    const float zp = __builtin_fmaf((float)((1024 >> P) + Codec<BITS>::kCentre), sm, sz);
+    const float2v w = {__builtin_fmaf((float)r.x, sp, -zp), __builtin_fmaf((float)r.y, sp, -zp)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));
+  } else {
+    const half2v u = centre_raw<P>(raw, Codec<BITS>::kCentre);
+    const float2v w = {__builtin_fmaf((float)u.x, sm, -sz), __builtin_fmaf((float)u.y, sm, -sz)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(w, bf16x2));
+  }
 }
 
 template <int BITS, int J>

@@ -237,7 +237,9 @@ def test_planner_splits_k_in_the_workgroup_where_ring_tiles_would_sit_one_per_cu
     assert _lib.describe_plan(4, 128, 10240, 8192, 512, True).endswith("cfg11")
     assert _lib.describe_plan(8, 128, 8192, 8192, 1024, True).endswith("cfg11")
     assert _lib.describe_plan(6, 128, 8192, 8192, 1024, True).endswith("cfg3")     # 6 bits: registers
-    assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True, 3).endswith("cfg3")  # bf16 likewise
+    assert _lib.describe_plan(3, 128, 8192, 8192, 1024, True, 3).endswith("cfg3")  # 3 bits on bf16 storage likewise
+    assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True, 3).endswith("cfg11")
+    assert _lib.describe_plan(8, 128, 8192, 8192, 1024, True, 3).endswith("cfg11")
     # short K walks as well, down to where the small staged tile fits one round
     assert _lib.describe_plan(4, 128, 4096, 2048, 1024, True).endswith("cfg10")
     assert _lib.describe_plan(4, 128, 4096, 1024, 1024, True).endswith("cfg10")
@@ -254,13 +256,24 @@ def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
     assert _lib.describe_plan(4, -1, 8192, 8192, 2048, True).endswith("cfg0")
 
 
-def test_planner_gives_bf16_storage_the_narrower_ring_tiles():
-    # bf16 weights are formed in fp32 (twice the vector work per weight): the 128 x 256 tile stalls
-    # on it; 128 x 192 where its rounds pay (not at 6 bits: registers), else 128 x 128.  Every tile can be forced.
-    assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3).endswith("cfg9")
-    assert _lib.describe_plan(4, 128, 57344, 8192, 2048, False, 3).endswith("cfg9")
-    assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 3).endswith("cfg3")
+def test_planner_gives_bf16_storage_the_wide_ring_tile_where_its_registers_hold():
+    # bf16 weights are formed in fp32 (four vector instructions per pair instead of three).  2- and 4-bit
+    # codes, and 8-bit codes with one scale per row, follow the rules of fp16 storage; the others spill in
+    # the 128 x 256 tile: 128 x 192 where its rounds pay (not at 6 bits: registers), else 128 x 128, and
+    # 8-bit codes the 128 x 256 tile split over eight waves up to two rounds of them.  Every tile can be forced.
+    for bits in (2, 4):
+        for zp in (True, False):
+            assert _lib.describe_plan(bits, 128, 10240, 8192, 2048, zp, 3) == _lib.describe_plan(bits, 128, 10240, 8192, 2048, zp, 1)
+            assert _lib.describe_plan(bits, 128, 57344, 8192, 2048, zp, 3).endswith("cfg0")
+            assert _lib.describe_plan(bits, -1, 8192, 28672, 2048, zp, 3).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 1024, True, 3).endswith("cfg9")
+    assert _lib.describe_plan(8, -1, 8192, 8192, 2048, True, 3).endswith("cfg0")
+    assert _lib.describe_plan(4, 32, 8192, 8192, 2048, False, 3).endswith("cfg3")
+    assert _lib.describe_plan(3, 128, 8192, 8192, 2048, True, 3).endswith("cfg3")
+    assert _lib.describe_plan(3, 128, 10240, 8192, 2048, True, 3).endswith("cfg9")
     assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True, 3).endswith("cfg9")
+    assert _lib.describe_plan(8, 128, 8192, 8192, 2048, True, 3).endswith("cfg11")
+    assert _lib.describe_plan(8, 128, 6144, 4096, 2048, True, 3).endswith("cfg9")
     assert _lib.describe_plan(6, 128, 57344, 8192, 2048, True, 3).endswith("cfg3")
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8)).endswith("cfg8")
 
