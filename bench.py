@@ -82,10 +82,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
-    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill", "midbatch", "medium"),
+    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill", "prefill_bf16", "midbatch", "medium"),
                     help="for rocprofv3 --pmc runs.  decode: launch only the dominant kernel over the ring of "
                          "weight copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's "
-                         "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer.  "
+                         "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer (prefill_bf16: on bf16 storage).  "
                          "midbatch: launch only the mid-batch kernel, 4096->4096 at M=64 and 14336->4096 at M=16.  "
                          "medium: launch only the ring tiles that split K inside the workgroup, 8192->8192 at "
                          "M=512 and M=1024")
@@ -154,17 +154,18 @@ def main() -> int:
         return sorted(times)[len(times) // 2]
 
     bits = 4
-    if args.counter_pass == "prefill":
+    if args.counter_pass in ("prefill", "prefill_bf16"):
         n, k = LLAMA3_70B["o"]
+        dt, fl = (torch.bfloat16, 3) if args.counter_pass == "prefill_bf16" else (torch.float16, 1)
         packed = make_ring(n, k, bits, 1)[0]
-        sc, zr = make_aux(n, k)
-        x = torch.randn(2048, k, device=dev, generator=g).to(torch.float16)
-        y = torch.empty(2048, n, dtype=torch.float16, device=dev)
+        sc, zr = (t.to(dt) for t in make_aux(n, k))
+        x = torch.randn(2048, k, device=dev, generator=g).to(dt)
+        y = torch.empty(2048, n, dtype=dt, device=dev)
         with torch.cuda.stream(stream):
             for _ in range(6):
-                launch(bits, n, k, x, packed, sc, zr, y)
+                launch(bits, n, k, x, packed, sc, zr, y, flags=fl)
             stream.synchronize()
-        print(json.dumps({"counter_pass": _lib.describe_plan(bits, GROUP, n, k, 2048, True), "launches": 6}))
+        print(json.dumps({"counter_pass": _lib.describe_plan(bits, GROUP, n, k, 2048, True, fl), "launches": 6}))
         return 0
     if args.counter_pass == "medium":
         n, k = LLAMA3_70B["o"]
