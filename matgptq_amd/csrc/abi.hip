@@ -276,20 +276,24 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   }
   // Batch rows 1..4: the gemv kernel (every wave requests a whole round of
   // tiles at once).  Measured on MI355X (Llama-3-8B layers, every bitwidth): four tiles per
-  // wave and round; one row block per workgroup at batch 1 and on layers with few row blocks,
-  // two above that (the staged activations of several batch rows are then shared); as many
+  // wave and round; one row block per workgroup at batch 1 and 2 and on layers with few row blocks,
+  // two above that (the staged activations of three or four batch rows are then shared); as many
   // waves as there are rounds of four tiles, sixteen at most.  2-bit tiles are half the bytes
   // for the same work per tile: with two row blocks per workgroup (one staging of the
   // activations for both) the 28672 x 4096 layer takes 7.7 instead of 8.4 us; the layers with
   // few row blocks lose that way (4096 x 14336: 6.4 against 5.0 us).
   // Group sizes 32 and -1 run the two shapes named here (a scale per octet, or per row).
   if (M <= kGemvMaxM && flavour == 0 && (variant == 0 || variant >= 100)) {
-    int shape = ((M >= 2 && row_blocks >= 320) || (bits == 2 && group_size == 128 && row_blocks >= 1024)) ? 2 : 1;
-    // several batch rows, 2 or 3 bits, many row blocks: four row blocks per workgroup share one
+    // (two batch rows have an instantiation of their own, which stages two rows where the one for
+    // three and four stages four: with it one row block per workgroup is ahead at M = 2 as well -
+    // 28672 x 4096: 4 bits 11.5 against 12.6 us, 6 bits 16.1 against 17.5, 3 bits 10.7 against 11.5 on the
+    // four-row-block shape)
+    int shape = ((M >= 3 && row_blocks >= 320) || (bits == 2 && group_size == 128 && row_blocks >= 1024)) ? 2 : 1;
+    // three or four batch rows, 2 or 3 bits, many row blocks: four row blocks per workgroup share one
     // staging of the activations and their codes still fit the registers of eight waves
     // per SIMD (28672 x 4096 at M = 4: 3 bits 11.8 against 13.1 us, 2 bits 9.35 against 10.0;
     // 4 bits 14.9 against 13.5: its 64 registers of codes leave four waves per SIMD)
-    if (M >= 2 && bits <= 3 && group_size == 128 && row_blocks >= 1024) shape = 6;
+    if (M >= 3 && bits <= 3 && group_size == 128 && row_blocks >= 1024) shape = 6;
     if (variant >= 100) {
       shape = variant - 100;
       if (shape >= kNumGemvShapes) return MATGPTQ_EVARIANT;

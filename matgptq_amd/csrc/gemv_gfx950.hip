@@ -71,8 +71,12 @@ __device__ __forceinline__ float quad_sum(float v) {
 // LDS bytes per wave: X' of one round for MB batch rows + a block of zeros (group 32: as long as
 // one batch row's X', so that tile offsets apply to it too) + group 32's table of octet sums
 constexpr int gemv_zero_bytes(int t, int group) { return group == 32 ? t * 256 : 256; }
+// bytes from one batch row's X' to the next: the four live lanes of an operand read take the
+// same 16 bytes of four different batch rows, which a stride of whole KiB would put into the
+// same banks
+constexpr int gemv_row_bytes(int t, int mb) { return t * 256 + (mb > 1 ? 16 : 0); }
 constexpr int gemv_wave_lds(int t, int mb, int group) {
-  return mb * t * 256 + gemv_zero_bytes(t, group) + (group == 32 ? mb * t * 32 : 0);
+  return mb * gemv_row_bytes(t, mb) + gemv_zero_bytes(t, group) + (group == 32 ? mb * t * 32 : 0);
 }
 
 // MASTER: `a.packed` holds master-resident bit planes (master_layout.h); the rounded slice to
@@ -85,7 +89,8 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
   constexpr int TH = (T + 3) / 4;  // groups of four tiles per round
   constexpr int NS = GROUP == 128 ? TH : GROUP == 32 ? T : 1;  // scale registers per row block
   constexpr float kMul = (float)(1 << (8 - BITS));
-  constexpr int kXBytes = MB * T * 256;
+  constexpr int kRowBytes = gemv_row_bytes(T, MB);
+  constexpr int kXBytes = MB * kRowBytes;
   constexpr int kZeroBytes = gemv_zero_bytes(T, GROUP);
   constexpr int kWaveBytes = gemv_wave_lds(T, MB, GROUP);
   extern __shared__ __align__(16) unsigned char smem[];
@@ -107,7 +112,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
   // activation operand: row n of A is batch row n % 4 while tile u = n / 4 of a group of four is
   // multiplied; the batch rows beyond M repeat row M - 1 (their results are never stored)
   const int arow = (n & 3) < a.M ? (n & 3) : a.M - 1;
-  const unsigned char* a_live = xw + (MB > 1 ? arow * T * 256 : 0) + q * 16;
+  const unsigned char* a_live = xw + (MB > 1 ? arow * kRowBytes : 0) + q * 16;
   const unsigned char* a_zero = xw + kXBytes + q * 16;
 
   float acc[R][MB];
@@ -196,7 +201,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         so = dot2(v.p[2], ones, so);
         so = dot2(v.p[3], ones, so);
         if (T >= 4 || 4 * h + q < T)
-          *reinterpret_cast<uint4*>(xw + m * T * 256 + h * 1024 + lane * 16) = v.v;
+          *reinterpret_cast<uint4*>(xw + m * kRowBytes + h * 1024 + lane * 16) = v.v;
         if constexpr (kPerOctet) {
           // sums over the four chunks of an octet; the first lane of the quad files them under
           // (batch row, tile 4 h + lane / 16, octet chunk / 4)
@@ -339,6 +344,9 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
   if (a.M == 1)
     return zp ? launch_shape<true, GROUP, 1, MASTER>(a, shape, W, lds_pad, stream)
               : launch_shape<false, GROUP, 1, MASTER>(a, shape, W, lds_pad, stream);
+  if (a.M == 2)
+    return zp ? launch_shape<true, GROUP, 2, MASTER>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, GROUP, 2, MASTER>(a, shape, W, lds_pad, stream);
   return zp ? launch_shape<true, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream)
             : launch_shape<false, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream);
 }

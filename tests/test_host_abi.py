@@ -165,6 +165,12 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(2, 128, 28672, 4096, 1, True) == "gemv b2 g128 zp1 T4 R2 W8 pad0"
     assert _lib.describe_plan(3, 128, 28672, 4096, 4, True) == "gemv b3 g128 zp1 T4 R4 W8 pad0"
     assert _lib.describe_plan(3, 128, 6144, 4096, 4, True) == "gemv b3 g128 zp1 T4 R2 W8 pad0"
+    # two batch rows stage two rows (three and four stage four): one row block per workgroup stays ahead,
+    # except for 2-bit tiles on layers with many rows
+    assert _lib.describe_plan(4, 128, 28672, 4096, 2, True) == "gemv b4 g128 zp1 T4 R1 W8 pad0"
+    assert _lib.describe_plan(3, 128, 28672, 4096, 2, True) == "gemv b3 g128 zp1 T4 R1 W8 pad0"
+    assert _lib.describe_plan(2, 128, 28672, 4096, 2, True) == "gemv b2 g128 zp1 T4 R2 W8 pad0"
+    assert _lib.describe_plan(4, 128, 28672, 4096, 3, True) == "gemv b4 g128 zp1 T4 R2 W8 pad0"
     assert _lib.describe_plan(4, 32, 4096, 4096, 5).startswith(("decode", "midbatch"))
     # five to sixteen rows: the mid-batch kernel, except at 8 bits on fp16 storage with one scale per
     # tile or row, on layers with many rows (two row blocks per workgroup only)
