@@ -54,7 +54,7 @@ extern "C" {
 #define MATGPTQ_FLAG_VARIANT_MASK 0xFF00u
 #define MATGPTQ_FLAG_FLAVOUR_SHIFT 16
 #define MATGPTQ_FLAG_FLAVOUR_MASK 0x30000u
-/* gemv kernel (batch 1..4, group 128; variant 100 + entry): bits 18..22 waves per workgroup
+/* gemv kernel (batch 1..4; 5..8 with one scale per tile or row, entries 1 and 2; variant 100 + entry): bits 18..22 waves per workgroup
  * (0 = automatic), bits 23..28 dynamic LDS to request, in units of 4 KiB (0 = what it needs) */
 #define MATGPTQ_FLAG_GEMV_WAVES_SHIFT 18
 #define MATGPTQ_FLAG_GEMV_LDS_SHIFT 23

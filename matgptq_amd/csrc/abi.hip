@@ -53,6 +53,7 @@ namespace {
 
 constexpr int kDecodeMaxM = 16;
 constexpr int kGemvMaxM = 4;
+constexpr int kGemvEightMaxM = 8;  // its instantiation for five to eight batch rows (group sizes 128 and -1)
 // (tiles per wave and round, row blocks per workgroup) of the gemv kernel's instantiations
 // (group sizes 32 and -1 and the master-resident planes: entries 1 and 2 only)
 constexpr int kNumGemvShapes = 7;
@@ -260,7 +261,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     }
   } else if (flavour == 0 && M > kGemvMaxM &&
              !(bits == 8 && group_size != 32 && !(flags & MATGPTQ_FLAG_BF16) && row_blocks >= 1024)) {
-    // Five to sixteen batch rows (one to four go to the gemv kernel below): every decode
+    // Five to sixteen batch rows (one to four go to the gemv kernel below, and five to eight on
+    // layers with few row blocks): every decode
     // workgroup stages the whole batch of activations (scaled copies, written by the vector
     // ALU), which grows with M and K, while the mid-batch kernel copies them into LDS
     // asynchronously.  Measured on MI355X (Llama-3-8B layers, 2, 4 and 8 bits, M = 5 .. 16, weights
@@ -283,7 +285,19 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   // activations for both) the 28672 x 4096 layer takes 7.7 instead of 8.4 us; the layers with
   // few row blocks lose that way (4096 x 14336: 6.4 against 5.0 us).
   // Group sizes 32 and -1 run the two shapes named here (a scale per octet, or per row).
-  if (M <= kGemvMaxM && flavour == 0 && (variant == 0 || variant >= 100)) {
+  // Five to eight batch rows on layers with few row blocks: there the mid-batch kernel has one
+  // workgroup per CU at most and is bound by the instructions it issues per tile; the gemv
+  // kernel's instantiation for eight batch rows (two tiles per chain of MFMAs) is ahead up to
+  // 512 row blocks - M = 8, 4 bits: 4096 x 14336 9.6 against 11.9 us, 4096 x 4096 4.4 against 5.3,
+  // 6144 x 4096 5.5 against 6.0 (two row blocks per workgroup from 320 row blocks on), 8192 x 28672 25.8
+  // against 29.5; 2, 3, 6 and 8 bits alike, except 6 bits on 512 row blocks (13.6 against 12.2).  Beyond
+  // (10240 x 8192: 16.5 against 14.9; 28672 x 4096: 18.5 against 16.5) the mid-batch kernel's four
+  // row blocks per staged activation tile win.
+  const bool eight_domain = M > kGemvMaxM && M <= kGemvEightMaxM && group_size != 32;
+  const bool eight_auto = eight_domain && variant == 0 &&
+                          (row_blocks < 320 || (row_blocks <= 512 && !(bits == 6 && row_blocks > 384)));
+  const bool gemv_eight = eight_domain && (variant >= 100 || eight_auto);
+  if ((M <= kGemvMaxM || gemv_eight) && flavour == 0 && (variant == 0 || variant >= 100)) {
     // (two batch rows have an instantiation of their own, which stages two rows where the one for
     // three and four stages four: with it one row block per workgroup is ahead at M = 2 as well -
     // 28672 x 4096: 4 bits 11.5 against 12.6 us, 6 bits 16.1 against 17.5, 3 bits 10.7 against 11.5 on the
@@ -294,18 +308,30 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     // per SIMD (28672 x 4096 at M = 4: 3 bits 11.8 against 13.1 us, 2 bits 9.35 against 10.0;
     // 4 bits 14.9 against 13.5: its 64 registers of codes leave four waves per SIMD)
     if (M >= 3 && bits <= 3 && group_size == 128 && row_blocks >= 1024) shape = 6;
+    if (M > kGemvMaxM) shape = row_blocks < 320 ? 1 : 2;
     if (variant >= 100) {
       shape = variant - 100;
       if (shape >= kNumGemvShapes) return MATGPTQ_EVARIANT;
-      if (group_size != 128 && shape != 1 && shape != 2) return MATGPTQ_EVARIANT;
+      if ((group_size != 128 || M > kGemvMaxM) && shape != 1 && shape != 2) return MATGPTQ_EVARIANT;
     }
     const int T = kGemvShapes[shape][0];
     int Wg = (int)((flags >> MATGPTQ_FLAG_GEMV_WAVES_SHIFT) & 31u);
+    const bool waves_given = Wg != 0;
     if (Wg == 0) {
       Wg = (k_tiles + T - 1) / T;
       if (Wg > 16) Wg = 16;
     }
     if (Wg > 16) return MATGPTQ_EVARIANT;
+    if (M > kGemvMaxM) {
+      // eight batch rows of X' per wave, the table of their sums, the zero block and the wave's
+      // partial sums: as many waves as fit the LDS of a CU
+      const int per_wave = 8 * (T * 256 + 16) + 256 + 8 * T * 8 + kGemvShapes[shape][1] * 4 * 256;
+      const int fit = 160 * 1024 / per_wave;
+      if (Wg > fit) {
+        if (waves_given) return MATGPTQ_EVARIANT;
+        Wg = fit;
+      }
+    }
     p->gemv = true;
     p->decode = false;
     p->skinny = false;
@@ -468,7 +494,10 @@ const char* matgptq_strerror(int code) {
 
 // The kernels that read master-resident bit planes themselves: the gemv kernel in its two shapes
 // built for them, and the mid-batch kernel.
-static bool plan_reads_planes(const Plan& p) { return (p.gemv && (p.shape == 1 || p.shape == 2)) || p.skinny; }
+// (the gemv kernel reads the planes up to four batch rows)
+static bool plan_reads_planes(const Plan& p, int64_t M) {
+  return (p.gemv && M <= kGemvMaxM && (p.shape == 1 || p.shape == 2)) || p.skinny;
+}
 
 // checks, plan, launch; `master_planes`: the weight operand is master-resident bit planes and
 // the plan must be one of those kernels (the caller has made sure of it)
@@ -482,7 +511,7 @@ static int run_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t 
   if (!weights_dev || !scales_dev || !x_dev || !y_dev) return MATGPTQ_ENULL;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &p)) return e;
-  if (master_planes && !plan_reads_planes(p)) return MATGPTQ_EVARIANT;
+  if (master_planes && !plan_reads_planes(p, M)) return MATGPTQ_EVARIANT;
   GemmArgs a;
   a.packed = static_cast<const uint32_t*>(weights_dev);
   a.scales = static_cast<const uint16_t*>(scales_dev);
@@ -530,12 +559,12 @@ static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t 
   if (M <= 0) return MATGPTQ_ESIZE;
   Plan p;
   if (int e = make_plan(bitwidth, group_size, N, K, M, zp, *flags, &p)) return e;
-  *direct = plan_reads_planes(p);
+  *direct = plan_reads_planes(p, M);
   const bool automatic = (*flags & MATGPTQ_FLAG_VARIANT_MASK) == 0 && ((*flags >> 16) & 3u) == 0;
   if (!*direct && automatic && M > kGemvMaxM && M <= 128) {
     const uint32_t msel = M <= 16 ? 0u : M <= 32 ? 1u : 2u;  // 16, 32 or 64 batch rows per workgroup
     const uint32_t forced = *flags | ((80u + 2u + 3u * msel) << MATGPTQ_FLAG_VARIANT_SHIFT);  // four row blocks, or as many as fit
-    if (make_plan(bitwidth, group_size, N, K, M, zp, forced, &p) == MATGPTQ_OK && plan_reads_planes(p)) {
+    if (make_plan(bitwidth, group_size, N, K, M, zp, forced, &p) == MATGPTQ_OK && plan_reads_planes(p, M)) {
       *flags = forced;
       *direct = true;
     }

@@ -75,9 +75,12 @@ constexpr int gemv_zero_bytes(int t, int group) { return group == 32 ? t * 256 :
 // same 16 bytes of four different batch rows, which a stride of whole KiB would put into the
 // same banks
 constexpr int gemv_row_bytes(int t, int mb) { return t * 256 + (mb > 1 ? 16 : 0); }
+// (eight batch rows: a table of the two sums per batch row and tile)
 constexpr int gemv_wave_lds(int t, int mb, int group) {
-  return mb * gemv_row_bytes(t, mb) + gemv_zero_bytes(t, group) + (group == 32 ? mb * t * 32 : 0);
+  return mb * gemv_row_bytes(t, mb) + gemv_zero_bytes(t, group) + (group == 32 ? mb * t * 32 : mb > 4 ? mb * t * 8 : 0);
 }
+// accumulators per lane and row block: the batch rows of one lane quarter
+constexpr int gemv_lane_rows(int mb) { return mb < 4 ? mb : 4; }
 
 // MASTER: `a.packed` holds master-resident bit planes (master_layout.h); the rounded slice to
 // BITS is formed in registers while the raw pairs are built.
@@ -87,7 +90,16 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
   constexpr bool kPerOctet = GROUP == 32;  // a scale per octet: the row groups of A take turns per octet
   static_assert(!kPerOctet || T <= 4, "one lane per 16 bytes of the zero block");
   constexpr int TH = (T + 3) / 4;  // groups of four tiles per round
-  constexpr int NS = GROUP == 128 ? TH : GROUP == 32 ? T : 1;  // scale registers per row block
+  // Up to four batch rows the sixteen rows of the activation operand are four tiles x four batch
+  // rows and a chain of MFMAs covers four tiles; five to eight batch rows make them two tiles x
+  // eight batch rows: a chain covers two tiles, lane (n, q) ends with tile q / 2, batch rows
+  // 4 (q % 2) .. + 3, and the sums of a tile travel through a small table in LDS.
+  constexpr bool kEight = MB > 4;
+  static_assert(!kEight || (!kPerOctet && T % 2 == 0), "eight batch rows: group sizes 128 and -1");
+  constexpr int TPC = kEight ? 2 : 4;              // tiles per chain
+  constexpr int NC = (T + TPC - 1) / TPC;          // chains per round
+  constexpr int NV = gemv_lane_rows(MB);           // accumulators per lane and row block
+  constexpr int NS = GROUP == 128 ? NC : GROUP == 32 ? T : 1;  // scale registers per row block
   constexpr float kMul = (float)(1 << (8 - BITS));
   constexpr int kRowBytes = gemv_row_bytes(T, MB);
   constexpr int kXBytes = MB * kRowBytes;
@@ -103,23 +115,26 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
   const int rb0 = blockIdx.x * R;
 
   unsigned char* xw = smem + wave * kWaveBytes;                   // this wave's X' and zeros
-  float* red = reinterpret_cast<float*>(smem + W * kWaveBytes);   // [W][R * MB][64]
+  float* red = reinterpret_cast<float*>(smem + W * kWaveBytes);   // [W][R * NV][64]
   if (lane * 16 < kZeroBytes) *reinterpret_cast<uint4*>(xw + kXBytes + lane * 16) = make_uint4(0, 0, 0, 0);
-  float2* const osum = reinterpret_cast<float2*>(xw + kXBytes + kZeroBytes);  // group 32: [MB][T][4] (off, xs)
+  float2* const osum = reinterpret_cast<float2*>(xw + kXBytes + kZeroBytes);  // group 32: [MB][T][4] (off, xs); eight batch rows: [MB][T]
 
   constexpr uint32_t tile_bytes = Fmt::kTileBytes;
   const typename Fmt::Consts consts;
   // activation operand: row n of A is batch row n % 4 while tile u = n / 4 of a group of four is
   // multiplied; the batch rows beyond M repeat row M - 1 (their results are never stored)
-  const int arow = (n & 3) < a.M ? (n & 3) : a.M - 1;
+  // (eight batch rows: row n is batch row n % 8 during tile n / 8 of a pair of tiles)
+  const int brow = kEight ? (n & 7) : (n & 3);
+  const int slot = kEight ? (n >> 3) : (n >> 2);
+  const int arow = brow < a.M ? brow : a.M - 1;
   const unsigned char* a_live = xw + (MB > 1 ? arow * kRowBytes : 0) + q * 16;
   const unsigned char* a_zero = xw + kXBytes + q * 16;
 
-  float acc[R][MB];
+  float acc[R][NV];
 #pragma unroll
   for (int rr = 0; rr < R; rr++)
 #pragma unroll
-    for (int v = 0; v < MB; v++) acc[rr][v] = 0.f;
+    for (int v = 0; v < NV; v++) acc[rr][v] = 0.f;
 
   for (int kt0 = wave * T; kt0 < a.k_tiles; kt0 += W * T) {
     const int left = a.k_tiles - kt0;
@@ -152,9 +167,10 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
       const BufRsrc zr = make_rsrc(ZP ? a.zeros : a.scales, rows ? s_end : 0u);
 #pragma unroll
       for (int h = 0; h < NS; h++) {
-        // lane (n, q): group 128, the scale of row n in tile 4 h + q; group 32, in octet q of tile h
-        const uint32_t lo = GROUP == -1 ? (uint32_t)n * 2u : (uint32_t)lane * 2u;
-        const uint32_t so = GROUP == -1 ? (uint32_t)(rb0 + rr) * 32u : (sg0 + 4 * h) * 32u;  // (group 32: h = tile)
+        // lane (n, q): group 128, the scale of row n in tile 4 h + q (eight batch rows: 2 h + q / 2);
+        // group 32, in octet q of tile h
+        const uint32_t lo = GROUP == -1 ? (uint32_t)n * 2u : kEight ? (uint32_t)((q >> 1) * 16 + n) * 2u : (uint32_t)lane * 2u;
+        const uint32_t so = GROUP == -1 ? (uint32_t)(rb0 + rr) * 32u : (sg0 + TPC * h) * 32u;  // (group 32: h = tile)
         sv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(sr, lo, so, 0);
         if constexpr (ZP) zv[rr][h] = __builtin_amdgcn_raw_buffer_load_b16(zr, lo, so, 0);
       }
@@ -202,7 +218,12 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         so = dot2(v.p[3], ones, so);
         if (T >= 4 || 4 * h + q < T)
           *reinterpret_cast<uint4*>(xw + m * kRowBytes + h * 1024 + lane * 16) = v.v;
-        if constexpr (kPerOctet) {
+        if constexpr (kEight) {
+          // the first lane of a quarter files the sums of its tile under (batch row, tile)
+          xs[m][h] = row_sum16(sx);
+          off[m][h] = 1024.0f * row_sum16(so);
+          if (n == 0 && 4 * h + q < T) osum[m * T + 4 * h + q] = make_float2(off[m][h], xs[m][h]);
+        } else if constexpr (kPerOctet) {
           // sums over the four chunks of an octet; the first lane of the quad files them under
           // (batch row, tile 4 h + lane / 16, octet chunk / 4)
           const float2 pair = make_float2(1024.0f * quad_sum(so), quad_sum(sx));
@@ -222,7 +243,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
     for (int rr = 0; rr < R; rr++) d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < T; i++) {
-      const int u = i & 3;
+      const int u = i & (TPC - 1);
       Frag av[4];
       if constexpr (kPerOctet) {
         // octet j: row group j live (the zero block is as long as X', so `i * 256` applies to both)
@@ -230,7 +251,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         for (int j = 0; j < 4; j++)
           av[j].v = *reinterpret_cast<const uint4*>(((n >> 2) == j ? a_live : a_zero) + i * 256 + j * 64);
       } else {
-        const unsigned char* ab = (n >> 2) == u ? a_live + i * 256 : a_zero;
+        const unsigned char* ab = slot == u ? a_live + i * 256 : a_zero;
 #pragma unroll
         for (int j = 0; j < 4; j++) av[j].v = *reinterpret_cast<const uint4*>(ab + j * 64);
       }
@@ -246,13 +267,17 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
         Fmt::template raw<3>(w[rr][i], consts, bw.u);
         d[rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[3].h, bw.h, d[rr], 0, 0, 0);
       }
-      if (kPerOctet || u == 3 || i == T - 1) {
+      if (kPerOctet || u == TPC - 1 || i == T - 1) {
         const int h = i >> 2;
-        const int si = GROUP == 128 ? h : GROUP == 32 ? i : 0;
-        float fo[MB], fx[MB];
+        const int si = GROUP == 128 ? i / TPC : GROUP == 32 ? i : 0;
+        float fo[NV], fx[NV];
 #pragma unroll
-        for (int v = 0; v < MB; v++) {
-          if constexpr (kPerOctet) {
+        for (int v = 0; v < NV; v++) {
+          if constexpr (kEight) {
+            const float2 pair = osum[((q & 1) * 4 + v) * T + (i / TPC) * TPC + (q >> 1)];
+            fo[v] = pair.x;
+            fx[v] = pair.y;
+          } else if constexpr (kPerOctet) {
             const float2 pair = osum[(v * T + i) * 4 + q];
             fo[v] = pair.x;
             fx[v] = pair.y;
@@ -267,26 +292,27 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
           float zs = (float)(1 << (BITS - 1));
           if constexpr (ZP) zs = storage_to_float(zv[rr][si]) * (1.0f / kMul);
 #pragma unroll
-          for (int v = 0; v < MB; v++) acc[rr][v] += s * (d[rr][v] - fo[v] - zs * fx[v]);
+          for (int v = 0; v < NV; v++) acc[rr][v] += s * (d[rr][v] - fo[v] - zs * fx[v]);
           d[rr] = float4v{0.f, 0.f, 0.f, 0.f};
         }
       }
     }
   }
 
-  // ---- the four lane quarters and the W waves meet: red[wave][rr * MB + v][lane]
+  // ---- the lane quarters that hold the same batch rows and the W waves meet: red[wave][rr * NV + v][lane]
 #pragma unroll
   for (int rr = 0; rr < R; rr++)
 #pragma unroll
-    for (int v = 0; v < MB; v++) red[((wave * R + rr) * MB + v) * 64 + lane] = acc[rr][v];
+    for (int v = 0; v < NV; v++) red[((wave * R + rr) * NV + v) * 64 + lane] = acc[rr][v];
   __syncthreads();
-  for (int o = wave; o < R * MB; o += W) {
+  for (int o = wave; o < R * NV; o += W) {
     float sum = 0.f;
-    for (int w2 = 0; w2 < W; w2++) sum += red[(w2 * R * MB + o) * 64 + lane];
-    sum += __shfl_xor(sum, 16);
+    for (int w2 = 0; w2 < W; w2++) sum += red[(w2 * R * NV + o) * 64 + lane];
+    if constexpr (!kEight) sum += __shfl_xor(sum, 16);
     sum += __shfl_xor(sum, 32);
-    const int rr = o / MB, v = o - rr * MB;
-    if (q == 0 && rb0 + rr < a.row_blocks && v < a.M)
+    const int rr = o / NV;
+    const int v = o - rr * NV + (kEight ? q * 4 : 0);  // batch row (eight: quarters 0 and 1 hold rows 0..3 and 4..7)
+    if (q < (kEight ? 2 : 1) && rb0 + rr < a.row_blocks && v < a.M)
       a.y[(size_t)v * a.N + (size_t)(rb0 + rr) * 16 + n] = float_to_storage(sum * kMul);
   }
 }
@@ -300,7 +326,7 @@ __global__ void __launch_bounds__(1024, WPE) gemv_kernel(const GemmArgs a, const
 template <bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER>
 hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stream) {
   const dim3 grid((a.row_blocks + R - 1) / R), block(64 * W);
-  size_t smem = (size_t)W * gemv_wave_lds(T, MB, GROUP) + (size_t)W * R * MB * 256;
+  size_t smem = (size_t)W * gemv_wave_lds(T, MB, GROUP) + (size_t)W * R * gemv_lane_rows(MB) * 256;
   if (smem < lds_pad) smem = lds_pad;
   if (W < 1 || W > 16 || a.M > MB || smem > 160 * 1024) return hipErrorInvalidValue;
   if (smem > 64 * 1024) {
@@ -321,7 +347,7 @@ hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stre
 // storage and the group sizes 32 and -1 take the two shapes the planner uses
 template <bool ZP, int GROUP, int MB, bool MASTER>
 hipError_t launch_shape(const GemmArgs& a, int shape, int W, size_t lds_pad, hipStream_t s) {
-  if constexpr (MASTER || GROUP != 128) {
+  if constexpr (MASTER || GROUP != 128 || MB > 4) {
     if (shape == 2) return launch_one<ZP, GROUP, 4, 2, MB, 4, MASTER>(a, W, lds_pad, s);
     if (shape == 1) return launch_one<ZP, GROUP, 4, 1, MB, 4, MASTER>(a, W, lds_pad, s);
     return hipErrorInvalidValue;
@@ -347,8 +373,14 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
   if (a.M == 2)
     return zp ? launch_shape<true, GROUP, 2, MASTER>(a, shape, W, lds_pad, stream)
               : launch_shape<false, GROUP, 2, MASTER>(a, shape, W, lds_pad, stream);
-  return zp ? launch_shape<true, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream)
-            : launch_shape<false, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream);
+  if (a.M <= 4)
+    return zp ? launch_shape<true, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream);
+  // five to eight batch rows: pre-sliced tiles with one scale per tile or row
+  if constexpr (GROUP != 32 && !MASTER)
+    return zp ? launch_shape<true, GROUP, 8, false>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, GROUP, 8, false>(a, shape, W, lds_pad, stream);
+  return hipErrorInvalidValue;
 }
 
 }  // namespace
@@ -356,7 +388,8 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 // Entry of this translation unit.  shape: index into the (T, R) table above; W: waves per
 // workgroup (1..16); lds_pad: dynamic LDS to ask for when it exceeds what the kernel needs
 // (limits how many workgroups share a CU); master: `a.packed` holds master-resident bit planes
-// (shapes 1 and 2); group sizes 32 and -1: shapes 1 and 2.  M <= 4 only.
+// (shapes 1 and 2); group sizes 32 and -1: shapes 1 and 2.  M <= 4; five to eight batch rows on
+// pre-sliced tiles with group size 128 or -1, shapes 1 and 2.
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 #if MATGPTQ_BF16

@@ -13,17 +13,18 @@ pytestmark = pytest.mark.gpu
 LLAMA8B = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "down": (4096, 14336)}
 LLAMA70B = {"qkv": (10240, 8192), "o": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
 
-# kernel the planner takes per layer and batch size (4 and 3 bits take the same, except that 3 bits
+# kernel the planner takes per layer and batch size (eight batch rows: the gemv kernel up to 512 row
+# blocks; 4 and 3 bits take the same, except that 3 bits
 # take four row blocks per workgroup on the layer with many rows at four batch rows: `{r}`)
 SMALL_BATCH_PLANS = {
     "qkv": {2: "gemv b{b} g128 zp1 T4 R1 W8 pad0", 4: "gemv b{b} g128 zp1 T4 R2 W8 pad0",
-            8: "midbatch b{b} g128 zp1 R2 mb1", 16: "midbatch b{b} g128 zp1 R2 mb1"},
+            8: "gemv b{b} g128 zp1 T4 R2 W8 pad0", 16: "midbatch b{b} g128 zp1 R2 mb1"},
     "o": {2: "gemv b{b} g128 zp1 T4 R1 W8 pad0", 4: "gemv b{b} g128 zp1 T4 R1 W8 pad0",
-          8: "midbatch b{b} g128 zp1 R1 mb1", 16: "midbatch b{b} g128 zp1 R1 mb1"},
+          8: "gemv b{b} g128 zp1 T4 R1 W8 pad0", 16: "midbatch b{b} g128 zp1 R1 mb1"},
     "gate_up": {2: "gemv b{b} g128 zp1 T4 R1 W8 pad0", 4: "gemv b{b} g128 zp1 T4 R{r} W8 pad0",
                 8: "midbatch b{b} g128 zp1 R4 mb1", 16: "midbatch b{b} g128 zp1 R4 mb1"},
     "down": {2: "gemv b{b} g128 zp1 T4 R1 W16 pad0", 4: "gemv b{b} g128 zp1 T4 R1 W16 pad0",
-             8: "midbatch b{b} g128 zp1 R1 mb1", 16: "midbatch b{b} g128 zp1 R1 mb1"},
+             8: "gemv b{b} g128 zp1 T4 R1 W16 pad0", 16: "midbatch b{b} g128 zp1 R1 mb1"},
 }
 
 

@@ -1,4 +1,5 @@
-"""The batch-1..4 kernel (gemv_gfx950.hip) against the oracle, through the C ABI.
+"""The batch-1..4 kernel (gemv_gfx950.hip), and its instantiation for five to eight batch rows,
+against the oracle, through the C ABI.
 
 Every instantiation (tiles per wave and round x row blocks per workgroup), every bitwidth,
 both zero-point forms, ragged row-block counts and ragged rounds of K tiles, both storage types,
@@ -92,8 +93,61 @@ def test_gemv_group_sizes_agree_with_the_decode_kernel():
             assert np.max(np.abs(a - c)) <= 2.0 ** -9 * np.max(np.abs(c))
 
 
+@pytest.mark.parametrize("g", (128, -1))
+@pytest.mark.parametrize("zp", (False, True))
+@pytest.mark.parametrize("b", BITS)
+def test_gemv_five_to_eight_batch_rows(b, zp, g):
+    # two tiles x eight batch rows in the activation operand, the sums of a tile through a table in
+    # LDS; 5 row blocks and 13 K tiles as above (ragged for two row blocks per workgroup, ragged rounds,
+    # an odd number of tiles: the last chain of MFMAs covers one tile)
+    n, k = 80, 128 * 13
+    lay = G.Layer(n, k, b, g, seed=40 + b, zero_points=zp)
+    for m in (5, 6, 7, 8):
+        x = o.make_activations(m, k, seed=m + b, outlier_frac=0.01)
+        assert _lib.describe_plan(b, g, n, k, m, zp).startswith("gemv")
+        G.assert_close_to_oracle(lay.run(x), x, lay.w, f"default b={b} g={g} zp={zp} M={m}")
+        for shape in (1, 2):
+            for waves in (0, 1, 3, 16):
+                if shape == 2 and waves == 16:  # more LDS than a CU has
+                    with pytest.raises(_lib.MatGPTQError, match="variant"):
+                        lay.run(x, flags=gemv_flags(shape, waves))
+                    continue
+                y = lay.run(x, flags=gemv_flags(shape, waves))
+                G.assert_close_to_oracle(y, x, lay.w, f"b={b} g={g} zp={zp} M={m} shape={shape} W={waves}")
+                G.assert_regression_bound(y, x, lay.w, f"b={b} g={g} zp={zp} M={m} shape={shape} W={waves}")
+
+
+def test_gemv_five_to_eight_batch_rows_long_k():
+    # 224 K tiles: several rounds per wave, fifteen waves with two row blocks per workgroup (LDS)
+    lay = G.Layer(64, 28672, 4, 128, seed=4)
+    x = o.make_activations(8, 28672, seed=8)
+    assert _lib.describe_plan(4, 128, 64, 28672, 8, True, gemv_flags(2)) == "gemv b4 g128 zp1 T4 R2 W15 pad0"
+    for shape in (1, 2):
+        y = lay.run(x, flags=gemv_flags(shape))
+        G.assert_close_to_oracle(y, x, lay.w, f"long K shape={shape}")
+        G.assert_regression_bound(y, x, lay.w, f"long K shape={shape}")
+
+
+def test_gemv_five_to_eight_batch_rows_exact_in_the_reference_test_regime():
+    rng = np.random.default_rng(5)
+    n, k = 48, 4096
+    for b in BITS:
+        codes = rng.integers(0, 1 << b, (n, k), dtype=np.uint8)
+        scales = np.round(rng.random((n, k // 128))).astype(np.float16)
+        pk = G.pack_device(codes, b, from_master=False)
+        sd = G.reorder_device(scales, n, k, 128)
+        w = o.dequantize_kernel_form(codes, scales, b, 128)
+        for m in (5, 8):
+            x = np.round(rng.standard_normal((m, k))).astype(np.float16)
+            expect = o.linear_f64(x, w).astype(np.float16)
+            for shape in (1, 2):
+                y = G.gemm(b, 128, n, k, G.to_dev(x), pk, sd, None, flags=gemv_flags(shape)).cpu().numpy()
+                assert np.array_equal(y.view(np.uint16), expect.view(np.uint16)), (b, m, shape)
+
+
 def test_gemv_is_not_taken_outside_its_domain():
-    assert _lib.describe_plan(4, 128, 4096, 4096, 5, True).split()[0] in ("decode-burst", "midbatch")
+    assert _lib.describe_plan(4, 128, 4096, 4096, 9, True).split()[0] in ("decode-burst", "midbatch")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 5, True).split()[0] in ("decode-burst", "midbatch")
     assert _lib.describe_plan(4, 32, 4096, 4096, 5, True).split()[0].startswith(("decode", "midbatch"))
     with pytest.raises(_lib.MatGPTQError, match="variant"):  # group 32: shapes 1 and 2 only
         G.Layer(32, 256, 4, 32, seed=1).run(o.make_activations(1, 256, seed=1), flags=gemv_flags(0))
@@ -185,12 +239,12 @@ def test_gemv_bf16_storage(b):
         return out
 
     sr, zr = reorder(s), reorder(z)
-    for m in (1, 4):
+    for m in (1, 4, 7):
         x = o.round_to_bf16(o.make_activations(m, k, seed=m + b, outlier_frac=0.01).astype(np.float32))
         xd = dev_bf16(x)
         for zeros, zz in ((zr, z), (None, np.full_like(z, 128.0))):
             ref = o.linear_f64(x, o.dequantize_bf16(q, s, zz, b, 128))
-            for shape in (1, 2, 4):
+            for shape in (1, 2, 4) if m <= 4 else (1, 2):
                 y = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=G.DEV)
                 _lib.check(L.matgptq_gemm(b, 128, n, k, m, pk.data_ptr(), sr.data_ptr(),
                                           zeros.data_ptr() if zeros is not None else None, xd.data_ptr(),

@@ -99,14 +99,17 @@ def test_midbatch_kernel_reads_the_planes_itself(b, g, m):
     planes = planes_device(q)
     sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
     x = o.make_activations(m, k, seed=m)
-    assert _lib.describe_plan(b, g, n, k, m, True).startswith("midbatch")
+    # (five to eight batch rows of a pre-sliced layer this small go to the gemv kernel, which reads the
+    # planes up to four: on planes they take the mid-batch kernel, forced here for the comparison)
+    flags = 1 | (82 << 8) if 5 <= m <= 8 and g != 32 else 1
+    assert _lib.describe_plan(b, g, n, k, m, True, flags).startswith("midbatch")
     for zeros in (zr, None):
         y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zeros, workspace=None)
         assert need == 0
         zz = z if zeros is not None else np.full_like(z, 128)
         G.assert_close_to_oracle(y, x, o.dequantize(q, s, zz, b, g), f"planes, mid-batch b={b} g={g} M={m}")
         # bit-identical to the pre-sliced tensor: the same codes reach the same arithmetic
-        y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zeros).cpu().numpy()
+        y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zeros, flags=flags).cpu().numpy()
         assert np.array_equal(y, y2)
 
 

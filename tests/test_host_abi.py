@@ -154,7 +154,7 @@ def test_error_codes():
 
 
 def test_describe_plan_regimes():
-    # batch 1..4: the gemv kernel; five rows on: decode / mid-batch
+    # batch 1..4: the gemv kernel; five rows on: decode / mid-batch, or the gemv kernel again (below)
     assert _lib.describe_plan(4, 128, 4096, 4096, 1) == "gemv b4 g128 zp0 T4 R1 W8 pad0"
     assert _lib.describe_plan(4, 128, 4096, 14336, 1, True) == "gemv b4 g128 zp1 T4 R1 W16 pad0"
     assert _lib.describe_plan(4, 128, 4096, 4096, 4, True) == "gemv b4 g128 zp1 T4 R1 W8 pad0"
@@ -182,7 +182,17 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(8, 128, 28672, 4096, 5, True).startswith("decode")
     assert _lib.describe_plan(8, -1, 28672, 4096, 16, False).startswith("decode")
     assert _lib.describe_plan(4, 128, 28672, 4096, 5, True) == "midbatch b4 g128 zp1 R4 mb1"
-    assert _lib.describe_plan(8, 128, 4096, 4096, 5, True) == "midbatch b8 g128 zp1 R1 mb1"
+    # five to eight rows on layers with at most 512 row blocks: the gemv kernel's instantiation for eight
+    # batch rows (one scale per tile or row; two row blocks per workgroup from 320 row blocks on)
+    assert _lib.describe_plan(8, 128, 4096, 4096, 5, True) == "gemv b8 g128 zp1 T4 R1 W8 pad0"
+    assert _lib.describe_plan(4, 128, 4096, 14336, 8, True) == "gemv b4 g128 zp1 T4 R1 W16 pad0"
+    assert _lib.describe_plan(4, -1, 6144, 4096, 6, False) == "gemv b4 g-1 zp0 T4 R2 W8 pad0"
+    assert _lib.describe_plan(4, 128, 8192, 28672, 8, True) == "gemv b4 g128 zp1 T4 R2 W15 pad0"  # (LDS: fifteen waves)
+    assert _lib.describe_plan(6, 128, 8192, 8192, 8, True) == "midbatch b6 g128 zp1 R2 mb1"
+    assert _lib.describe_plan(6, 128, 6144, 4096, 8, True) == "gemv b6 g128 zp1 T4 R2 W8 pad0"
+    assert _lib.describe_plan(4, 128, 10240, 8192, 8, True).startswith("midbatch")
+    assert _lib.describe_plan(4, 128, 4096, 4096, 9, True) == "midbatch b4 g128 zp1 R1 mb1"
+    assert _lib.describe_plan(8, 32, 4096, 4096, 5, True) == "midbatch b8 g32 zp1 R1 mb1"
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048).startswith("prefill")
     with pytest.raises(RuntimeError):
         _lib.describe_plan(4, 128, 4096, 4096, 1, True, 1 | (107 << 8))   # no such gemv entry
@@ -193,7 +203,7 @@ def test_describe_plan_regimes():
     assert _lib.describe_plan(8, 128, 28672, 4096, 16, True).startswith("decode")
     assert _lib.describe_plan(4, 128, 28672, 4096, 16, True) == "midbatch b4 g128 zp1 R4 mb1"
     # small layers: the mid-batch kernel (K split inside the workgroup) from a few rows on
-    assert _lib.describe_plan(4, 128, 4096, 4096, 8, True).startswith("midbatch")
+    assert _lib.describe_plan(4, 128, 4096, 4096, 16, True).startswith("midbatch")
     assert _lib.describe_plan(4, 32, 4096, 14336, 5, True).startswith("midbatch")
     assert _lib.describe_plan(3, 32, 16, 1024, 17).startswith("midbatch")
     assert _lib.describe_plan(4, 128, 4096, 4096, 128, True) == "midbatch b4 g128 zp1 R4 mb2"
