@@ -320,3 +320,39 @@ def test_header_is_plain_c(tmp_path):
     src.write_text('#include "matgptq_abi.h"\nint main(void) { return matgptq_abi_version() == 0; }\n')
     subprocess.run([cc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
                     "-c", str(src), "-o", str(tmp_path / "t.o")], check=True)
+
+
+def test_planner_answers_every_valid_shape_within_its_kernels_domains():
+    # seeded random problems: a plan for each, the gemv kernel only up to eight batch rows (five to
+    # eight: one scale per tile or row, at most 512 row blocks, waves within the LDS of a CU), the
+    # mid-batch kernel from five rows on, the large-batch tiles from seventeen
+    import random
+    import re
+    rnd = random.Random(7)
+    seen = set()
+    for _ in range(6000):
+        b = rnd.choice((2, 3, 4, 6, 8))
+        g = rnd.choice((128, 32, -1))
+        n = 16 * rnd.choice((1, 2, 5, 16, 64, 255, 256, 319, 320, 384, 512, 513, 640, 1024, 1792, 3584, 8016))
+        k = 128 * rnd.choice((1, 2, 3, 4, 7, 8, 16, 31, 32, 64, 112, 224)) + (64 if g != 128 and rnd.random() < 0.1 else 0)
+        m = rnd.choice((1, 2, 3, 4, 5, 6, 7, 8, 9, 15, 16, 17, 31, 32, 33, 64, 100, 128, 129, 256, 384, 512, 1000, 1024, 2048, 4096))
+        flags = 1 | (2 if rnd.random() < 0.3 else 0)
+        if k % 128 == 64 and k < 192:
+            continue
+        plan = _lib.describe_plan(b, g, n, k, m, rnd.random() < 0.5, flags)
+        kind = plan.split()[0]
+        seen.add(kind)
+        if kind == "gemv":
+            assert m <= 8, plan
+            w, r, t = (int(re.search(rf" {c}(\d+)", plan).group(1)) for c in "WRT")
+            assert 1 <= w <= 16, plan
+            if m > 4:
+                assert g != 32 and n // 16 <= 512, plan
+                assert w * (8 * (t * 256 + 16) + 256 + 64 * t + r * 1024) <= 160 * 1024, plan
+        elif kind == "midbatch":
+            assert m > 4, plan
+        elif kind == "prefill":
+            assert m > 16, plan
+        else:
+            assert kind.startswith("decode") and m <= 16, plan
+    assert {"gemv", "midbatch", "prefill"} <= seen
