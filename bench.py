@@ -82,11 +82,13 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
-    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "prefill", "prefill_bf16", "midbatch", "medium"),
+    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "small", "prefill", "prefill_bf16", "midbatch", "medium"),
                     help="for rocprofv3 --pmc runs.  decode: launch only the dominant kernel over the ring of "
                          "weight copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's "
                          "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer (prefill_bf16: on bf16 storage).  "
                          "midbatch: launch only the mid-batch kernel, 4096->4096 at M=64 and 14336->4096 at M=16.  "
+                         "small: launch only the gemv kernel's instantiations for two and for eight batch rows, "
+                         "4096->28672 at M=2 and 14336->4096 at M=8.  "
                          "medium: launch only the ring tiles that split K inside the workgroup, 8192->8192 at "
                          "M=512 and M=1024")
     args = ap.parse_args()
@@ -182,9 +184,9 @@ def main() -> int:
             plans.append(f"M={m}: " + _lib.describe_plan(bits, GROUP, n, k, m, True))
         print(json.dumps({"counter_pass": plans, "launches_each": 6}))
         return 0
-    if args.counter_pass == "midbatch":
+    if args.counter_pass in ("midbatch", "small"):
         plans = []
-        for name, m in (("o", 64), ("down", 16)):
+        for name, m in ((("o", 64), ("down", 16)) if args.counter_pass == "midbatch" else (("gate_up", 2), ("down", 8))):
             n, k = LLAMA3_8B[name]
             copies = 16
             ring = make_ring(n, k, bits, copies)
