@@ -16,7 +16,9 @@ The JSON line also carries
                average launch duration measured with HIP events on the launch stream
   cpu_baseline the reference's PyTorch CPU path (slice -> dequantize -> F.linear,
                restated in oracle/torch_path.py) on the host cores, same layers, one pass
-  extra        per-bitwidth / per-layer times, small-batch and M=2048 prefill figures
+  summary      a dozen scalars of the tables below
+The per-bitwidth / per-layer / small-batch / M=2048 prefill tables go to gpurun_out/bench_extra.json
+and to stderr, one table per line; the last stdout line stays under 4 KB.
 """
 from __future__ import annotations
 
@@ -579,14 +581,75 @@ def main() -> int:
         # ---------------------------------------------------------- CPU baseline
         cpu_baseline = cpu_path_baseline(step_bytes)
 
+    headline = {"value": round(value, 1), "steps": args.steps, "warmup": args.warmup,
+                "ms_per_step": round(ms_per_step, 5), "wall_s_timed_region": round(t_wall, 4)}
+    extra_path = write_tables({"headline": headline, "roofline": roofline, "cpu_baseline": cpu_baseline, **extra})
+    print(final_line(headline, roofline, cpu_baseline, extra, extra_path))
+    return 0
+
+
+EXTRA_FILE = os.path.join("gpurun_out", "bench_extra.json")
+LINE_LIMIT = 4096  # bytes: the last stdout line has to fit the tail a harness keeps of the output
+
+
+def write_tables(tables: dict):
+    """The per-layer / per-bitwidth / per-batch tables go to a side file (and, one table per line, to
+    stderr); only scalars ride in the last stdout line.  Returns the file's path relative to the
+    repository root, or None when it cannot be written."""
+    for name, table in tables.items():
+        print(json.dumps({name: table}), file=sys.stderr)
+    try:
+        os.makedirs(os.path.join(ROOT, os.path.dirname(EXTRA_FILE)), exist_ok=True)
+        with open(os.path.join(ROOT, EXTRA_FILE), "w") as f:
+            json.dump(tables, f, indent=1)
+        return EXTRA_FILE
+    except OSError:
+        return None
+
+
+def final_line(headline: dict, roofline: dict, cpu_baseline, extra: dict, extra_path=None) -> str:
+    """The ONE JSON line that ends stdout: the contract's keys, `roofline`, `cpu_baseline` and a dozen
+    scalars picked from the tables.  Kept under LINE_LIMIT bytes whatever the tables hold."""
+    def pick(table, row, field):
+        try:
+            return extra[table][row][field]
+        except (KeyError, TypeError):
+            return None
+
+    floor = extra.get("read_floor") or {}
+    summary = {
+        "step_over_four_bare_reads": floor.get("step_measured_over_floor"),
+        "dominant_kernel_over_its_bare_read": floor.get("dominant_kernel_over_its_read"),
+        "four_bare_reads_us": floor.get("step_of_four_reads_us"),
+    }
+    for name in ("qkv", "o", "gate_up", "down"):
+        summary[f"gemv_b4_{name}_us"] = pick("gemv_M1", f"{name}_b4_zp", "us")
+    for b in (2, 3, 6, 8):
+        summary[f"gemv_b{b}_gate_up_pct_hbm_peak"] = pick("gemv_M1", f"gate_up_b{b}_zp", "pct_hbm_peak")
+    for name in ("qkv", "o", "gate_up", "down"):
+        summary[f"prefill_b4_M2048_{name}_pct_mfma_peak"] = pick("prefill_llama3_70b", f"{name}_b4_M2048_zp", "pct_mfma_peak")
+    wide = [v["pct_mfma_peak"] for r, v in (extra.get("prefill_llama3_70b") or {}).items()
+            if ("_b6_" in r or "_b8_" in r) and "pct_mfma_peak" in v]
+    summary["prefill_b6_b8_min_pct_mfma_peak"] = min(wide) if wide else None
+    medium = [v["speedup"] for v in (extra.get("medium_batch_llama3_70b_b4") or {}).values() if "speedup" in v]
+    summary["medium_batch_min_speedup_over_dense_fp16"] = min(medium) if medium else None
+    summary["decoder_tokens_per_s_graph"] = (extra.get("mixnmatch_decoder_end_to_end") or {}).get("tokens_per_s_graph")
+    summary["transformers_tokens_per_s_compiled"] = (extra.get("transformers_end_to_end") or {}).get("tokens_per_s_compiled")
+    summary = {k: v for k, v in summary.items() if v is not None}
+
+    roof = {k: roofline.get(k) for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel",
+                                         "us_per_launch", "algorithmic_bytes")}
+    cpu = None
+    if cpu_baseline is not None:
+        cpu = {k: cpu_baseline.get(k) for k in ("value", "unit", "cores", "kind", "sample")}
     out = {
         "metric": "batch1_gemv_sliced_weight_GBps_4bit_llama3_8b_layers",
-        "value": round(value, 1),
+        "value": headline["value"],
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
+        "steps": headline["steps"],
+        "warmup": headline["warmup"],
+        "ms_per_step": headline["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -594,14 +657,18 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": "configs[1]: Llama-3-8B linears qkv/o/gate_up/down, M=1 decode, 4-bit slice, "
                                "group 128, fp16 scale+zero; ring of weight copies > 2 GiB",
-                   "pct_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 1),
-                   "wall_s_timed_region": round(t_wall, 4)},
-        "roofline": roofline,
-        "cpu_baseline": cpu_baseline,
-        "extra": extra,
+                   "pct_hbm_peak": round(headline["value"] / HBM_PEAK_GBPS * 100, 1),
+                   "wall_s_timed_region": headline["wall_s_timed_region"]},
+        "roofline": roof,
+        "cpu_baseline": cpu,
+        "summary": summary,
+        "tables": extra_path,
     }
-    print(json.dumps(out))
-    return 0
+    line = json.dumps(out)
+    if len(line) > LINE_LIMIT:  # never let the scalars push the contract's keys out of a kept tail
+        out["summary"] = {}
+        line = json.dumps(out)
+    return line
 
 
 def cpu_path_baseline(step_bytes: int):
