@@ -561,6 +561,16 @@ static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t 
   if (int e = make_plan(bitwidth, group_size, N, K, M, zp, *flags, &p)) return e;
   *direct = plan_reads_planes(p, M);
   const bool automatic = (*flags & MATGPTQ_FLAG_VARIANT_MASK) == 0 && ((*flags >> 16) & 3u) == 0;
+  if (!*direct && automatic && M <= kGemvMaxM) {
+    // the planner's own gemv shape for this problem has no instantiation on planes (four row blocks
+    // per workgroup at 2 and 3 bits): the two-row-block shape, which has one, serves every batch of
+    // one to four rows
+    const uint32_t forced = *flags | ((100u + 2u) << MATGPTQ_FLAG_VARIANT_SHIFT);
+    if (make_plan(bitwidth, group_size, N, K, M, zp, forced, &p) == MATGPTQ_OK && plan_reads_planes(p, M)) {
+      *flags = forced;
+      *direct = true;
+    }
+  }
   if (!*direct && automatic && M > kGemvMaxM && M <= 128) {
     const uint32_t msel = M <= 16 ? 0u : M <= 32 ? 1u : 2u;  // 16, 32 or 64 batch rows per workgroup
     const uint32_t forced = *flags | ((80u + 2u + 3u * msel) << MATGPTQ_FLAG_VARIANT_SHIFT);  // four row blocks, or as many as fit
@@ -574,9 +584,15 @@ static int master_reads_planes(int bitwidth, int group_size, int64_t N, int64_t 
 
 size_t matgptq_gemm_master_workspace_bytes(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
                                            uint32_t flags) {
-  bool direct = false;
-  if (master_reads_planes(bitwidth, group_size, N, K, M, true, &flags, &direct) != MATGPTQ_OK) return 0;
-  return direct ? 0 : matgptq_packed_words(bitwidth, N, K) * 4;
+  // The plan can depend on whether the call brings zero points: the workspace covers both forms, so
+  // that a size asked for once per layer holds for either call.
+  for (int zp = 0; zp < 2; ++zp) {
+    bool direct = false;
+    uint32_t f = flags;
+    if (master_reads_planes(bitwidth, group_size, N, K, M, zp != 0, &f, &direct) != MATGPTQ_OK) return 0;
+    if (!direct) return matgptq_packed_words(bitwidth, N, K) * 4;
+  }
+  return 0;
 }
 
 static int gemm_master_impl(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
@@ -609,6 +625,8 @@ int matgptq_gemm_master(int bitwidth, int group_size, int64_t N, int64_t K, int6
 
 // Address of this GPU's copy of `scratch`: looked up once per device, with that device current
 // (the array's name is only a host-side handle, not a device address).
+// The current device has to be the one that owns the call's stream (as for every entry point here:
+// the kernels are launched on the current device's copy of the code object).
 static int static_scratch(void** ptr) {
   constexpr int kMaxDevices = 64;
   static std::mutex lock;

@@ -31,6 +31,8 @@
 // tile leave its four octet sums side by side, lane (n, q) holds the scale and zero of octet q
 // (again one 2-byte load per lane, now per tile), and the per-octet sums  off  and  xs  travel
 // through a small table in LDS (a rotate-reduce over the 4 lanes of an octet fills it).
+#include <atomic>
+
 #include "tile_format.h"
 
 #ifndef MATGPTQ_BITS
@@ -330,13 +332,17 @@ hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stre
   if (smem < lds_pad) smem = lds_pad;
   if (W < 1 || W > 16 || a.M > MB || smem > 160 * 1024) return hipErrorInvalidValue;
   if (smem > 64 * 1024) {
-    // more than 64 KiB of dynamic LDS has to be allowed once per kernel
-    static bool allowed = false;
-    if (!allowed) {
+    // more than 64 KiB of dynamic LDS has to be allowed once per kernel and device (the attribute
+    // belongs to the device's copy of the code object): one bit per device, set after the call succeeded
+    static std::atomic<uint64_t> allowed{0};
+    int dev = 0;
+    if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (dev >= 64 || !(allowed.load(std::memory_order_acquire) & bit)) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
-      allowed = true;
+      if (dev < 64) allowed.fetch_or(bit, std::memory_order_release);
     }
   }
   hipLaunchKernelGGL((gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER>), grid, block, smem, stream, a, W);

@@ -124,3 +124,38 @@ def test_error_codes():
     assert lib.matgptq_gemm_master(4, 128, 4096, 4096, 2048, 1, 1, None, 1, 1, None, 0, None, 1) == -9
     assert lib.matgptq_gemm_master(4, 128, 4096, 4096, 2048, 1, 1, None, 1, 1, 1, 100, None, 1) == -9
     assert "workspace" in lib.matgptq_strerror(-9).decode()
+
+
+def test_batches_of_one_to_four_rows_never_need_a_workspace():
+    """Whatever gemv shape the planner prefers on pre-sliced codes (four row blocks per workgroup at
+    2 and 3 bits on layers with many rows has no instantiation on planes), a call on planes with one
+    to four batch rows reads them in the kernel."""
+    lib = L()
+    for bits in (2, 3, 4, 6, 8):
+        for g in (128, 32, -1):
+            for n, k in ((4096, 4096), (6144, 4096), (28672, 4096), (4096, 14336), (57344, 8192), (128256, 4096)):
+                if bits * n * k // 8 >= 1 << 32 or n * k >= 1 << 32:
+                    continue
+                for m in (1, 2, 3, 4):
+                    assert lib.matgptq_gemm_master_workspace_bytes(bits, g, n, k, m, 1) == 0, (bits, g, n, k, m)
+    # the case that used to fall back to slicing 44 MB per call
+    assert lib.matgptq_gemm_master_workspace_bytes(3, 128, 28672, 4096, 3, 0) == 0
+
+
+def test_workspace_size_covers_the_call_with_and_without_zero_points():
+    """The planner's choice can depend on whether zero points are passed; the size covers both.
+    b = 2, g = 32, 18128 x 31872 at M = 182: mid-batch kernel with zero points, the 128 x 256 tile
+    split over eight waves (which needs the sliced tensor) without."""
+    lib = L()
+    bits, g, n, k, m = 2, 32, 18128, 31872, 182
+    need = lib.matgptq_gemm_master_workspace_bytes(bits, g, n, k, m, 1)
+    assert need == bits * n * k // 8
+    described = {zp: _describe(lib, bits, g, n, k, m, zp) for zp in (0, 1)}
+    assert described[1].startswith("midbatch") and described[0].startswith("prefill"), described
+
+
+def _describe(lib, bits, g, n, k, m, zp, flags=1):
+    import ctypes
+    buf = ctypes.create_string_buffer(128)
+    assert lib.matgptq_describe_plan(bits, g, n, k, m, zp, flags, buf, 128) == 0
+    return buf.value.decode()
