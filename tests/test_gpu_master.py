@@ -254,3 +254,20 @@ def test_master_gemm_in_a_graph():
             graph.replay()
             stream.synchronize()
             assert torch.equal(out4, eager[4]) and torch.equal(out3, eager[3])
+
+
+@pytest.mark.parametrize("b,m", [(3, 3), (2, 4), (3, 4), (2, 3)])
+def test_three_and_four_rows_on_many_row_layers_read_the_planes(b, m):
+    # the pre-sliced plan here is the gemv kernel with four row blocks per workgroup, which is not built
+    # for planes: on planes the two-row-block shape serves the call, without a workspace
+    n, k, g = 16384, 512, 128
+    assert "R4" in _lib.describe_plan(b, g, n, k, m, True)
+    q, s, z = o.make_layer(n, k, g, seed=b * 7 + m)
+    planes = planes_device(q)
+    sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
+    x = o.make_activations(m, k, seed=m)
+    for zeros in (zr, None):
+        y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zeros, workspace=None)
+        assert need == 0
+        zz = z if zeros is not None else np.full_like(z, 128)
+        G.assert_close_to_oracle(y, x, o.dequantize(q, s, zz, b, g), f"planes, gemv R2 b={b} M={m}")
