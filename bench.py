@@ -452,6 +452,15 @@ def main() -> int:
         from matgptq_amd import decoder
         extra["mixnmatch_decoder_end_to_end"] = decoder.measure(layers=32, context=512, new_tokens=64)
         torch.cuda.empty_cache()
+        # ---------------- the reference's transformers caller (inference_lib/bench_transformers_e2e.py):
+        # a LlamaForCausalLM of the same shape with MatGPTQLinear modules, StaticCache,
+        # torch.compile(fullgraph, reduce-overhead), timed like its time_prof
+        try:
+            from matgptq_amd import hf_bench
+            extra["transformers_end_to_end"] = hf_bench.measure(layers=32, context=512)
+        except Exception as e:  # transformers or the inductor toolchain absent: the figure is optional
+            extra["transformers_end_to_end"] = {"error": f"{type(e).__name__}: {str(e)[:200]}"}
+        torch.cuda.empty_cache()
         # --------------------------------------------------------------- prefill
         pre = {}
         m = 2048
