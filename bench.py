@@ -452,15 +452,6 @@ def main() -> int:
         from matgptq_amd import decoder
         extra["mixnmatch_decoder_end_to_end"] = decoder.measure(layers=32, context=512, new_tokens=64)
         torch.cuda.empty_cache()
-        # ---------------- the reference's transformers caller (inference_lib/bench_transformers_e2e.py):
-        # a LlamaForCausalLM of the same shape with MatGPTQLinear modules, StaticCache,
-        # torch.compile(fullgraph, reduce-overhead), timed like its time_prof
-        try:
-            from matgptq_amd import hf_bench
-            extra["transformers_end_to_end"] = hf_bench.measure(layers=32, context=512)
-        except Exception as e:  # transformers or the inductor toolchain absent: the figure is optional
-            extra["transformers_end_to_end"] = {"error": f"{type(e).__name__}: {str(e)[:200]}"}
-        torch.cuda.empty_cache()
         # --------------------------------------------------------------- prefill
         pre = {}
         m = 2048
@@ -586,6 +577,15 @@ def main() -> int:
         load["host_slice_pack_b4_4096x4096"] = {"ms": round(best * 1e3, 2), "Mcodes_per_s": round(4096 * 4096 / best / 1e6, 1),
                                                 "threads": os.cpu_count()}
         extra["load_time"] = load
+        torch.cuda.empty_cache()
+        # ---------------- the reference's transformers caller (inference_lib/bench_transformers_e2e.py):
+        # a LlamaForCausalLM of the same shape with MatGPTQLinear modules, StaticCache,
+        # torch.compile(fullgraph, reduce-overhead), timed like its time_prof
+        try:
+            from matgptq_amd import hf_bench
+            extra["transformers_end_to_end"] = hf_bench.measure(layers=32, context=512)
+        except Exception as e:  # transformers or the inductor toolchain absent: the figure is optional
+            extra["transformers_end_to_end"] = {"error": f"{type(e).__name__}: {str(e)[:200]}"}
         torch.cuda.empty_cache()
         # ---------------------------------------------------------- CPU baseline
         cpu_baseline = cpu_path_baseline(step_bytes)
