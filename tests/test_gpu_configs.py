@@ -164,6 +164,52 @@ def test_config3_llama3_8b_block_through_the_plugin():
         G.assert_close_to_oracle(y, x, w, f"block linear {name} b={bits[f'blocks.0.{name}']}")
 
 
+def test_config3_full_size_decoder_graph_replays_and_every_distinct_linear():
+    # configs[3] as stated: 32 blocks of Llama-3-8B's shape, vocabulary 128256, context 512, batch 1,
+    # every linear at a seeded bitwidth from {2,3,4,6,8}, built through the vLLM quantisation method.
+    # (i) eight decode steps replayed from the HIP graph equal the same steps run eagerly, logits and
+    # tokens bit for bit; (ii) one linear of every distinct (shape, bitwidth) pair against the oracle
+    # at batch 1.
+    from matgptq_amd import decoder as D
+
+    cfg = D.DecoderConfig()
+    assert (cfg.hidden, cfg.ffn, cfg.layers, cfg.heads, cfg.kv_heads, cfg.vocab) == (4096, 14336, 32, 32, 8, 128256)
+    context = 512
+    dec, bits, masters = D.random_mixnmatch_decoder(cfg, context + 24, (2, 3, 4, 6, 8), seed=0, keep_master=True,
+                                                    via_plugin=True)
+    assert len(bits) == 128 and set(bits.values()) == {2, 3, 4, 6, 8}
+    prompt = torch.randint(0, cfg.vocab, (context,), device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
+    eager = D.DecodeSession(dec)
+    eager.prefill(prompt)
+    graphed = D.DecodeSession(dec)
+    graphed.prefill(prompt)
+    assert torch.isfinite(eager.logits).all()
+    assert torch.equal(eager.logits, graphed.logits)
+    graphed.capture()
+    for i in range(8):
+        eager.step()
+        graphed.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(eager.logits, graphed.logits), f"replay {i}"
+        assert torch.equal(eager.token, graphed.token), f"replay {i}"
+        assert int(graphed.pos.item()) == context + 1 + i
+    del eager, graphed
+    seen = set()
+    for full, b in bits.items():
+        _, blk, name = full.split(".")
+        if (name, b) in seen:
+            continue
+        seen.add((name, b))
+        codes, scale, zero = masters[full]
+        n, k = codes.shape
+        x = o.make_activations(1, k, seed=b + n % 89)
+        y = getattr(dec.blocks[int(blk)], name)(torch.from_numpy(x).cuda()).cpu().numpy()
+        ref, bound = G.oracle_product_in_chunks(codes.cpu().numpy(), scale.cpu().numpy(), zero.cpu().numpy(), b,
+                                                cfg.group_size, x)
+        G.assert_close_to_reference(y, ref, bound, f"configs[3] {full} b={b}")
+    assert len(seen) >= 16  # 4 shapes x 5 bitwidths, nearly all of them drawn among 128 linears
+
+
 def test_prefill_zero_point_form_deviation_per_weight():
     # The prefill kernels' zero-point form computes fma(c - 2^(b-1), scale 2^(8-b), -fp16(scale (zero - 128)))
     # while dequantize() rounds scale * fp16((c << (8-b)) - zero) once.  Bound of the difference per
