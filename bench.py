@@ -84,10 +84,12 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip the extra sweeps and the CPU baseline")
-    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "small", "prefill", "prefill_bf16", "midbatch", "medium"),
+    ap.add_argument("--counter-pass", nargs="?", const="decode", default=None, choices=("decode", "decode_b2", "decode_b3", "small", "prefill", "prefill_b6", "prefill_b8", "prefill_bf16", "midbatch", "medium"),
                     help="for rocprofv3 --pmc runs.  decode: launch only the dominant kernel over the ring of "
                          "weight copies, eagerly, then a plain elementwise copy of 256 MiB (the counter's "
-                         "yardstick).  prefill: launch only the M=2048 kernel of the 8192->8192 layer (prefill_bf16: on bf16 storage).  "
+                         "yardstick); decode_b2 / decode_b3: the same at 2 and 3 bits.  "
+                         "prefill: launch only the M=2048 kernel of the 8192->8192 layer (prefill_bf16: on bf16 storage; "
+                         "prefill_b6 / prefill_b8: 6-bit and 8-bit codes).  "
                          "midbatch: launch only the mid-batch kernel, 4096->4096 at M=64 and 14336->4096 at M=16.  "
                          "small: launch only the gemv kernel's instantiations for two and for eight batch rows, "
                          "4096->28672 at M=2 and 14336->4096 at M=8.  "
@@ -158,6 +160,9 @@ def main() -> int:
         return sorted(times)[len(times) // 2]
 
     bits = 4
+    if args.counter_pass in ("decode_b2", "decode_b3", "prefill_b6", "prefill_b8"):
+        bits = int(args.counter_pass[-1])
+        args.counter_pass = args.counter_pass[:-3]
     if args.counter_pass in ("prefill", "prefill_bf16"):
         n, k = LLAMA3_70B["o"]
         dt, fl = (torch.bfloat16, 3) if args.counter_pass == "prefill_bf16" else (torch.float16, 1)

@@ -99,10 +99,14 @@ __device__ __forceinline__ void refill_octet(BufRsrc rs, uint32_t tile_off, int 
 // KS = 2 (ring tiles only): a workgroup of eight waves, two groups of four that each walk one
 // half of K on the same tile with a ring of their own, so that a layer whose tiles number no more
 // than the CUs still runs two waves per SIMD; the second group's sums pass through LDS at the end.
-template <int BITS, int GROUP, bool ZP, int RBW, int MT, int KS = 1>
+// PAIR (ring tiles only): a workgroup of eight waves again, but each group of four owns a tile of its
+// own (tiles 2 lid and 2 lid + 1, the whole of K, a ring each): two plain workgroups in one, for
+// kernels whose other workgroups need eight waves.  A tile index from `lid_limit` on is empty.
+template <int BITS, int GROUP, bool ZP, int RBW, int MT, int KS = 1, bool PAIR = false>
 __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_tiles, int rb_base,
-                                             _Float16* lds) {
+                                             _Float16* lds, int lid_limit = 0x7fffffff) {
   static_assert(KS == 1 || (KS == 2 && prefill_lean(RBW, MT)), "K is split inside the ring tiles only");
+  static_assert(!PAIR || (KS == 1 && prefill_lean(RBW, MT)), "paired tiles are ring tiles with the whole of K each");
   constexpr int TM = 16 * MT;
   constexpr int GPT = GROUP == 32 ? 4 : 1;
   constexpr int XCHUNKS = TM * (kXs / 8) / 256;  // 16-byte chunks per thread per stage
@@ -113,12 +117,13 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile offsets stay scalar
-  const int wave = KS == 1 ? wave_wg : (wave_wg & 3);  // within its group of four
-  const int grp = KS == 1 ? 0 : (wave_wg >> 2);
+  const int wave = KS == 1 && !PAIR ? wave_wg : (wave_wg & 3);  // within its group of four
+  const int grp = KS == 1 && !PAIR ? 0 : (wave_wg >> 2);
+  if constexpr (PAIR) lid = 2 * lid + grp;
   // K tiles [k_lo, k_hi) in kt_n trips (the same count for both groups: they share the barriers; a
   // tile beyond k_hi reads as zeros)
   const int kt_n = KS == 1 ? a.k_tiles : (a.k_tiles + 1) / 2;
-  const int k_lo = grp * kt_n;
+  const int k_lo = KS == 1 ? 0 : grp * kt_n;
   const int k_hi = KS == 1 || grp == 1 ? a.k_tiles : kt_n;
   lds += grp * prefill_lds_halves(RBW, MT);
   const int r16 = lane & 15;
@@ -127,7 +132,8 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
   const int nt = lid / m_tiles;
   const int mtile = lid - nt * m_tiles;
   const int m0 = mtile * TM;
-  const int rb_first = rb_base + (nt * 4 + wave) * RBW;
+  // (an empty tile: every row block out of range, so nothing is fetched and nothing stored)
+  const int rb_first = lid < lid_limit ? rb_base + (nt * 4 + wave) * RBW : a.row_blocks;
 
   constexpr uint32_t tile_bytes = (uint32_t)tile_words(BITS) * 4;
   const uint32_t rb_bytes = (uint32_t)a.k_tiles * tile_bytes;
@@ -456,6 +462,8 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
   #pragma unroll
       for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
       // one tile; ra / rb: the rings of its two half tiles, rn: the ring of the next tile's first
+      // (measured and not adopted: one barrier per tile, in front of its last step, with the tile after
+      // next requested into both rings behind it - 1.5 to 2 % slower at M = 2048 on every layer)
       auto dtile = [&](int kb, uint32_t (&wc)[RBW][BITS], uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT],
                        _Float16* ra, _Float16* rb, _Float16* rn) {
         dstep(wc, sc, zc, J0{}, ra, 1);
@@ -690,6 +698,33 @@ prefill_tail_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
     prefill_body<BITS, GROUP, ZP, 2, 8>(a, blockIdx.x - n_big, m_tiles, rb_tail, lds);
 }
 
+// The same split of the weight rows in workgroups of eight waves: the 128 x 256 tiles two to a
+// workgroup (PAIR), and the 128 x 128 tiles of the remaining rows one to a workgroup whose two
+// groups of four waves take one half of K each.  The narrow tiles then number at most the CUs and
+// still run two waves per SIMD, where the kernel above leaves them one.
+template <int BITS, int GROUP, bool ZP>
+__global__ void __launch_bounds__(512, 2)
+prefill_tail8_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
+  __shared__ __align__(16) _Float16 lds[2 * prefill_lds_halves(4, 8)];
+  const int n_pairs = (n_big + 1) / 2;
+  if ((int)blockIdx.x < n_pairs)
+    prefill_body<BITS, GROUP, ZP, 4, 8, 1, true>(a, blockIdx.x, m_tiles, 0, lds, n_big);
+  else
+    prefill_body<BITS, GROUP, ZP, 2, 8, 2>(a, blockIdx.x - n_pairs, m_tiles, rb_tail, lds);
+}
+
+template <int GROUP, bool ZP>
+hipError_t launch_tail8(const GemmArgs& a, hipStream_t stream) {
+  const int m_tiles = (a.M + 127) / 128;
+  const int nb = prefill_tail_big_tiles(a.row_blocks, m_tiles);
+  const int rb_tail = nb * 16;
+  const int n_small = (a.row_blocks - rb_tail + 7) / 8;
+  const int n_big = nb * m_tiles;
+  const dim3 grid((n_big + 1) / 2 + n_small * m_tiles), block(512);
+  hipLaunchKernelGGL((prefill_tail8_kernel<kBits, GROUP, ZP>), grid, block, 0, stream, a, m_tiles, n_big, rb_tail);
+  return hipGetLastError();
+}
+
 template <int GROUP, bool ZP>
 hipError_t launch_tail(const GemmArgs& a, hipStream_t stream) {
   const int m_tiles = (a.M + 127) / 128;
@@ -723,6 +758,10 @@ hipError_t launch_split(const GemmArgs& a, hipStream_t stream) {
 
 template <int GROUP, bool ZP>
 hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
+#ifdef MATGPTQ_EXPERIMENT  // one instantiation only: quick compiles while tuning the ring loop
+  if constexpr (GROUP == 128 && ZP) return launch_cfg<GROUP, ZP, 4, 8>(a, s);
+  else return hipErrorInvalidValue;
+#else
   switch (cfg) {
     case 10: return launch_split<GROUP, ZP, 2, 8>(a, s);  // 128 x 128, K split in the workgroup
     case 11: return launch_split<GROUP, ZP, 4, 8>(a, s);  // 128 x 256, K split in the workgroup
@@ -735,8 +774,10 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 6: return launch_cfg<GROUP, ZP, 8, 2>(a, s);   // 32 x 512
     case 8: return launch_tail<GROUP, ZP>(a, s);        // 128 x 256, then a tail of 128 x 128
     case 9: return launch_cfg<GROUP, ZP, 3, 8>(a, s);   // 128 x 192
+    case 12: return launch_tail8<GROUP, ZP>(a, s);      // 128 x 256 in pairs, then a tail of 128 x 128 with K split
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
+#endif
 }
 
 }  // namespace

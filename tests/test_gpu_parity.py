@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(12))
+@pytest.mark.parametrize("cfg", range(13))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -308,11 +308,30 @@ def test_llama3_70b_layer_prefill_full_size():
     assert np.max(np.abs(y1.astype(np.float64) - y[5:6])) <= 2e-3 * np.max(np.abs(y1.astype(np.float64)))
 
 
+@pytest.mark.parametrize("zp", (True, False))
+def test_prefill_paired_tiles_with_a_split_tail_odd_tile_count(zp):
+    # 128 x 256 tiles two to a workgroup of eight waves, the remaining rows as 128 x 128 tiles with K
+    # split inside the workgroup: 73 activation tiles x 7 whole weight tiles = 511 wide tiles (the last
+    # workgroup's second tile is empty), 8 row blocks in the tail, ragged M
+    n, k, m = 1920, 384, 73 * 128 - 5
+    flags = 1 | ((64 + 12) << 8)
+    lay = G.Layer(n, k, 4, 128, seed=12, zero_points=zp)
+    x = o.make_activations(m, k, seed=12)
+    y = lay.run(x, flags=flags)
+    G.assert_close_to_oracle(y, x, lay.w, "paired tiles + split tail")
+    G.assert_regression_bound(y, x, lay.w, "paired tiles + split tail")
+    # the wide tiles run the four-wave tail kernel's arithmetic; the narrow ones add two halves of K
+    y8 = lay.run(x, flags=1 | ((64 + 8) << 8))
+    assert np.array_equal(y[:, :1792], y8[:, :1792])
+    assert np.max(np.abs(y[:, 1792:].astype(np.float64) - y8[:, 1792:])) <= 2e-3 * np.max(np.abs(y8.astype(np.float64)))
+
+
 def test_llama3_70b_qkv_prefill_full_size_with_tail_tiles():
-    # 10240 rows at M = 2048: the planner splits the launch into 128 x 256 tiles (rows below 8192)
-    # and a tail of 128 x 128 tiles; rows of both parts against the oracle
+    # 10240 rows at M = 2048: the planner splits the launch into 128 x 256 tiles (rows below 8192, two
+    # to a workgroup of eight waves) and a tail of 128 x 128 tiles with K split inside the workgroup;
+    # rows of both parts against the oracle
     n, k, m = 10240, 8192, 2048
-    assert _lib.describe_plan(4, 128, n, k, m, True).endswith("cfg8")
+    assert _lib.describe_plan(4, 128, n, k, m, True).endswith("cfg12")
     lay = G.Layer(n, k, 4, 128, seed=0)
     x = o.make_activations(m, k, seed=0)
     y = lay.run(x)

@@ -216,7 +216,7 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     # 640 tiles of 128 x 256 are one round of 512 resident workgroups and a quarter: the rows of
     # the quarter go to narrower tiles; whole rounds, or more than half a round left over, keep the
     # plain tile
-    assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True).endswith("cfg8")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True).endswith("cfg12")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 57344, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
@@ -304,7 +304,7 @@ def test_planner_keeps_six_bit_codes_off_the_largest_ring_tile():
     assert _lib.describe_plan(8, 128, 57344, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(8, 128, 57344, 8192, 2048, False).endswith("cfg0")
     assert _lib.describe_plan(8, 128, 8192, 8192, 2048, True).endswith("cfg0")
-    assert _lib.describe_plan(8, 128, 10240, 8192, 2048, True).endswith("cfg8")
+    assert _lib.describe_plan(8, 128, 10240, 8192, 2048, True).endswith("cfg12")
     assert _lib.describe_plan(8, 128, 8192, 8192, 2048, False).endswith("cfg0")
     assert _lib.describe_plan(3, 128, 8192, 8192, 2048, True).endswith("cfg0")
 
