@@ -151,7 +151,9 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       const int m_tiles = (int)((M + 127) / 128);
       const int nb = prefill_tail_big_tiles(row_blocks, m_tiles);
       const int64_t rest = (int64_t)((row_blocks - nb * 16 + 15) / 16) * m_tiles;
-      if (nb > 0 && rest > 0 && rest <= 256) p->cfg = 8;
+      // (one whole round only: behind three rounds the plain tile's fourth, half empty, costs less than
+      // the narrow tiles do - 57344 x 8192 at M = 1024: 752 against 771 us)
+      if (nb > 0 && rest > 0 && rest <= 256 && (int64_t)nb * m_tiles <= 512) p->cfg = 8;
       // When those narrow tiles number no more than the CUs, workgroups of eight waves do better: the
       // wide tiles two to a workgroup, each narrow tile with K split over two groups of four waves, so
       // that the last part of the launch runs two waves per SIMD as well (10240 x 8192 at M = 2048:
@@ -190,6 +192,15 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         const double t_128 = rounds(wgs_128);
         p->cfg = t_192 < t_128 && fits_192 ? 9 : 3;
         if (p->cfg == 3 && bf16 && bits == 8 && group_size != 32 && wgs_big <= 512) p->cfg = 11;
+        // 6-bit codes on fp16 storage with one scale per tile or row: one register set refilled octet by
+        // octet fits the 128 x 256 tile once the compiler is left to order the step itself (243 registers;
+        // with the ordering hints of the other widths it spilled).  Its four instructions per pair of
+        // weights keep it at 41-43 % of peak, just ahead of the narrower tiles where its tiles fill whole
+        // rounds (M = 2048: 8192 x 8192 263 against 265 us, 8192 x 28672 890 against 923).
+        if (bits == 6 && !bf16 && group_size != 32) {
+          const double t_256 = rounds(wgs_big) * 2.0 * 0.97;
+          if (t_256 < t_128 && (p->cfg == 3 || t_256 < t_192)) p->cfg = 0;
+        }
       } else if (wgs_192 <= 512 && fits_192) {
         // Fewer than 512 of the 128 x 256 tiles leave half of the CUs with one workgroup where the
         // kernel is built for two; 128 x 192 tiles that still fit one round of 512 spread the same
@@ -237,6 +248,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       } else if (wgs_big <= 256 && bits != 6 && !(bf16 && (bits == 3 || group_size == 32)) && !(group_size == 32 && zp)) {
         const double t = 5.0 + kt * (wgs_big > 192 ? 1.65 : 1.4);
         if (t < best) { best = t; p->cfg = 11; }
+        // the same with 128 x 192 tiles where those fill more of the CUs in their one round
+        // (10240 x 8192 at M = 512: 216 workgroups, 91 us against 94 on 160 of the wider tile)
+        const int64_t wgs_192s = ((N + 191) / 192) * ((M + 127) / 128);
+        const double t3 = 4.0 + kt * (wgs_192s > 192 ? 1.36 : 1.22);
+        if (wgs_192s <= 256 && t3 < best) { best = t3; p->cfg = 13; }
       }
       for (int mb = 2; mb <= (M > 32 ? 4 : 2); mb <<= 1) {
         const int64_t m_tiles = (M + 16 * mb - 1) / (16 * mb);
@@ -360,7 +376,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       R = 1 << ((variant - 80) % 3);
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
-      if (variant - 64 > 12) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 13) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 64;

@@ -347,6 +347,8 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       constexpr int kRest = (RBW - RBW / 2) * MT;        // ... of the second (one more row block when RBW is odd)
       constexpr int kValuHalf = (RBW / 2) * 26;          // vector instructions of the first half's row blocks, roughly
       constexpr int kValuRest = (RBW - RBW / 2) * 26;
+#ifndef MATGPTQ_NO_GROUPS
+      if constexpr (BITS != 6) {
       __builtin_amdgcn_sched_group_barrier(0x002, kValuHalf, 0);
 #pragma unroll
       for (int n = 0; n < kHalf; n++) {
@@ -358,6 +360,8 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         if (n & 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+      }
+#endif
       __builtin_amdgcn_sched_barrier(0);
     };
     using J0 = std::integral_constant<int, 0>;
@@ -775,6 +779,7 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 8: return launch_tail<GROUP, ZP>(a, s);        // 128 x 256, then a tail of 128 x 128
     case 9: return launch_cfg<GROUP, ZP, 3, 8>(a, s);   // 128 x 192
     case 12: return launch_tail8<GROUP, ZP>(a, s);      // 128 x 256 in pairs, then a tail of 128 x 128 with K split
+    case 13: return launch_split<GROUP, ZP, 3, 8>(a, s);  // 128 x 192, K split in the workgroup
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 #endif

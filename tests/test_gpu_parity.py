@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(13))
+@pytest.mark.parametrize("cfg", range(14))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -142,7 +142,7 @@ def test_prefill_split_tiles_every_format(b, g, zp):
     n, k, m = 304, 128 * 7, 200
     lay = G.Layer(n, k, b, g, seed=29 * b + (g & 7), zero_points=zp)
     x = o.make_activations(m, k, seed=b + 2)
-    for cfg in (10, 11):
+    for cfg in (10, 11, 13):
         flags = 1 | ((64 + cfg) << 8)
         for _ in range(2):
             G.assert_close_to_oracle(lay.run(x, flags=flags), x, lay.w, f"split tile cfg{cfg} b={b} g={g} zp={zp}")
@@ -150,7 +150,7 @@ def test_prefill_split_tiles_every_format(b, g, zp):
 
 
 @pytest.mark.parametrize("k_tiles", (1, 2, 3, 10))
-@pytest.mark.parametrize("cfg", (10, 11))
+@pytest.mark.parametrize("cfg", (10, 11, 13))
 def test_prefill_split_tiles_short_and_even_walks(cfg, k_tiles):
     # one K tile leaves the second group with nothing but zeros; two give each group a single trip
     n, k, m = 528, 128 * k_tiles, 130
@@ -165,7 +165,7 @@ def test_prefill_split_tile_agrees_with_the_plain_tile_closely():
     lay = G.Layer(n, k, 4, 128, seed=8)
     x = o.make_activations(m, k, seed=9)
     plain = lay.run(x, flags=1 | (67 << 8)).astype(np.float64)
-    for cfg in (10, 11):
+    for cfg in (10, 11, 13):
         y = lay.run(x, flags=1 | ((64 + cfg) << 8)).astype(np.float64)
         assert np.max(np.abs(y - plain)) <= 2.0 ** -9 * np.max(np.abs(plain))
         assert np.mean(y == plain) > 0.9

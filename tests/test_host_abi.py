@@ -250,7 +250,9 @@ def test_planner_splits_k_in_the_workgroup_where_ring_tiles_would_sit_one_per_cu
     assert _lib.describe_plan(4, 128, 8192, 8192, 512, True, 3).endswith("cfg10")  # bf16 storage too
     # more of those than CUs but at most as many 128 x 256 tiles: the wide tile, split
     assert _lib.describe_plan(4, 128, 8192, 8192, 1024, True).endswith("cfg11")
-    assert _lib.describe_plan(4, 128, 10240, 8192, 512, True).endswith("cfg11")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 768, True).endswith("cfg11")
+    # 128 x 192 tiles, split the same way, where they put more of the CUs to work in the one round
+    assert _lib.describe_plan(4, 128, 10240, 8192, 512, True).endswith("cfg13")
     assert _lib.describe_plan(8, 128, 8192, 8192, 1024, True).endswith("cfg11")
     assert _lib.describe_plan(6, 128, 8192, 8192, 1024, True).endswith("cfg3")     # 6 bits: registers
     assert _lib.describe_plan(3, 128, 8192, 8192, 1024, True, 3).endswith("cfg3")  # 3 bits on bf16 storage likewise
@@ -294,10 +296,13 @@ def test_planner_gives_bf16_storage_the_wide_ring_tile_where_its_registers_hold(
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True, 3 | (72 << 8)).endswith("cfg8")
 
 
-def test_planner_keeps_six_bit_codes_off_the_largest_ring_tile():
-    # 6-bit codes spill in the 128 x 256 tile; 8-bit codes keep one set there, refilled octet by octet
-    assert _lib.describe_plan(6, 128, 8192, 8192, 2048, True).endswith("cfg3")
-    assert _lib.describe_plan(6, 128, 28672 // 4, 8192, 2048, False).endswith("cfg3")
+def test_planner_six_and_eight_bit_codes_on_the_ring_tiles():
+    # 6- and 8-bit codes keep one register set on the 128 x 256 tile, refilled octet by octet; 6-bit codes
+    # take it where its tiles fill whole rounds (fp16 storage, one scale per tile or row)
+    assert _lib.describe_plan(6, 128, 8192, 8192, 2048, True).endswith("cfg0")
+    assert _lib.describe_plan(6, 128, 28672 // 4, 8192, 2048, False).endswith("cfg0")
+    assert _lib.describe_plan(6, 32, 8192, 8192, 2048, False).endswith("cfg3")
+    assert _lib.describe_plan(6, 128, 8192, 8192, 2048, True, 3).endswith("cfg3")  # bf16 storage: registers
     assert _lib.describe_plan(6, 128, 10240, 8192, 2048, False).endswith("cfg9")  # 54 tiles of 192 rows: two rounds
     # many rounds: the 128 x 192 tile, which still fits the registers
     assert _lib.describe_plan(6, 128, 57344, 8192, 2048, True).endswith("cfg9")
