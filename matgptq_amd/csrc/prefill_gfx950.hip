@@ -347,8 +347,10 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       constexpr int kRest = (RBW - RBW / 2) * MT;        // ... of the second (one more row block when RBW is odd)
       constexpr int kValuHalf = (RBW / 2) * 26;          // vector instructions of the first half's row blocks, roughly
       constexpr int kValuRest = (RBW - RBW / 2) * 26;
+      // The ordering hints pay 1 % at 2, 3 and 4 bits.  The wide codes go without: 6-bit codes spill
+      // with them (88 registers on the 128 x 256 tile), 8-bit codes run 0 to 2 % faster left alone.
 #ifndef MATGPTQ_NO_GROUPS
-      if constexpr (BITS != 6) {
+      if constexpr (BITS != 6 && BITS != 8) {
       __builtin_amdgcn_sched_group_barrier(0x002, kValuHalf, 0);
 #pragma unroll
       for (int n = 0; n < kHalf; n++) {

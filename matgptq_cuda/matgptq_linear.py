@@ -31,34 +31,34 @@ class MatGPTQLinear(torch.nn.Module):
     def __init__(self, qweight: torch.Tensor, scales: torch.Tensor, bitwidth: int, group_size: int,
                  zeros: Optional[torch.Tensor] = None, perm: Optional[torch.Tensor] = None):
         super().__init__()
-        self.n_out_features: int = qweight.shape[0]
-        self.n_in_features: int = qweight.shape[1]
-        self.bitwidth: int = bitwidth
-        self.group_size: int = group_size
+        n_out, n_in = qweight.shape
+        self.n_out_features, self.n_in_features = int(n_out), int(n_in)
+        self.bitwidth, self.group_size = bitwidth, group_size
+        # the storage type of the scales decides the arithmetic type of the layer (flag bit 1)
+        flag = MatGTPQ_FeatureFlags.ASYNC
+        if scales.dtype == torch.bfloat16:
+            flag = flag | MatGTPQ_FeatureFlags.IS_BF16
+        self.flag: int = int(flag)
 
-        self.flag: int = MatGTPQ_FeatureFlags.ASYNC + MatGTPQ_FeatureFlags.IS_BF16 * (scales.dtype == torch.bfloat16)
+        ops = torch.ops.matgptq_cuda
+        shape = (self.n_out_features, self.n_in_features)
 
-        self.matgptq_qweight = torch.nn.Parameter(
-            torch.ops.matgptq_cuda.pack_matgptq_qweights(
-                qweight, self.n_out_features, self.n_in_features, self.bitwidth, self.group_size, self.flag),
-            requires_grad=False)
-        self.matgptq_scales = torch.nn.Parameter(
-            torch.ops.matgptq_cuda.reorder_matgptq_scales(
-                scales, self.n_out_features, self.n_in_features, self.group_size),
-            requires_grad=False)
-        if zeros is not None:
-            self.matgptq_zeros = torch.nn.Parameter(
-                torch.ops.matgptq_cuda.reorder_matgptq_scales(
-                    zeros.to(scales.dtype).contiguous(), self.n_out_features, self.n_in_features, self.group_size),
-                requires_grad=False)
+        def frozen(t: torch.Tensor) -> torch.nn.Parameter:
+            return torch.nn.Parameter(t, requires_grad=False)
+
+        def per_group(t: torch.Tensor) -> torch.Tensor:  # scales and zeros share one device layout
+            return ops.reorder_matgptq_scales(t, *shape, self.group_size)
+
+        self.matgptq_qweight = frozen(ops.pack_matgptq_qweights(qweight, *shape, self.bitwidth, self.group_size, self.flag))
+        self.matgptq_scales = frozen(per_group(scales))
+        self.matgptq_zeros = None if zeros is None else frozen(per_group(zeros.to(scales.dtype).contiguous()))
+        if perm is None:
+            self.matgptq_perm = None
         else:
-            self.matgptq_zeros = None
-        if perm is not None:
             if perm.numel() != self.n_in_features:
                 raise ValueError("perm must have n_in_features elements")
-            self.register_buffer("matgptq_perm", perm.to(device=self.matgptq_qweight.device, dtype=torch.int64).reshape(-1))
-        else:
-            self.matgptq_perm = None
+            self.register_buffer("matgptq_perm",
+                                 perm.to(device=self.matgptq_qweight.device, dtype=torch.int64).reshape(-1))
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor) -> torch.Tensor:
