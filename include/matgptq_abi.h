@@ -39,6 +39,7 @@ extern "C" {
 #define MATGPTQ_ESIZE (-8)     /* a size exceeds what the entry point supports */
 #define MATGPTQ_EWORKSPACE (-9) /* workspace missing or too small */
 #define MATGPTQ_ESTATIC (-10)   /* needs more than the library's built-in workspace */
+#define MATGPTQ_EALIAS (-11)    /* an output buffer overlaps an input that other workgroups still read */
 
 /* feature_flag bits: the reference's `Features` word
  * (inference_lib/matgptq_cuda/csrc/include/common.cuh:78-86,
@@ -130,6 +131,28 @@ int matgptq_slice_device(const uint8_t *master_dev, int64_t count, int bitwidth,
 int matgptq_dequantize_device(int bitwidth, int group_size, int64_t N, int64_t K,
                               const void *packed_dev, const void *scales_dev,
                               const void *zeros_dev, void *w_dev, void *stream);
+
+/* ---- decode with the operator in front of the linear fused into it ---------------------
+ * No counterpart in the reference, whose callers run these as separate element-wise kernels between
+ * the linears (the transformers model of inference_lib/inference_demo_transformers.py:132-175; each
+ * costs a launch and a round trip through memory, more than a decode GEMV of the smaller layers).
+ * matgptq_gemm with the activations formed while the kernel stages them; fp16 storage, group size
+ * 128, 1 <= M <= 4 (the batch-1..4 kernel), pre-sliced codes:
+ *   MATGPTQ_PRE_SILU_MUL     a_dev is [M, 2K] (gate | up, as the fused gate_up linear leaves them):
+ *                            x = fp16(silu(gate)) * up, the roundings of two element-wise operators;
+ *                            b_dev, w_dev, out_dev unused.
+ *   MATGPTQ_PRE_ADD_RMSNORM  a_dev is the residual stream h [M, K], b_dev what is added to it [M, K]
+ *                            (or NULL), w_dev the norm's weight [K]:  v = h + b (one fp16 rounding),
+ *                            x = fp16(v * rsqrt(mean(v^2) + eps) * w);  v is also written to out_dev
+ *                            [M, K] when that is not NULL.  out_dev must not overlap a_dev or b_dev
+ *                            (MATGPTQ_EALIAS): other workgroups still read them.  K <= 8192.
+ * Shapes outside these limits return MATGPTQ_EVARIANT: run the operator and matgptq_gemm separately. */
+#define MATGPTQ_PRE_SILU_MUL 1
+#define MATGPTQ_PRE_ADD_RMSNORM 2
+int matgptq_gemm_prologue(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                          const void *packed_dev, const void *scales_dev, const void *zeros_dev,
+                          int kind, const void *a_dev, const void *b_dev, const void *w_dev, void *out_dev,
+                          float eps, void *y_dev, void *stream, uint32_t flags);
 
 /* Measurement aid (no counterpart in the reference): streams `bytes` of device memory once through
  * the load pattern of the batch-1 kernel (a wave requests four KiB-sized pieces at once, eight

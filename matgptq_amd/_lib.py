@@ -17,7 +17,7 @@ FLAG_BF16 = 2
 VARIANT_SHIFT = 8
 
 EXPORTS = (
-    "matgptq_abi_version", "matgptq_strerror", "matgptq_packed_words", "matgptq_gemm",
+    "matgptq_abi_version", "matgptq_strerror", "matgptq_packed_words", "matgptq_gemm", "matgptq_gemm_prologue",
     "matgptq_pack_host", "matgptq_unpack_host", "matgptq_reorder_scales_host",
     "matgptq_pack_device", "matgptq_unpack_device", "matgptq_reorder_scales_device",
     "matgptq_slice_device", "matgptq_dequantize_device", "matgptq_describe_plan",
@@ -51,6 +51,8 @@ def load() -> ctypes.CDLL:
     L.matgptq_packed_words.restype = ctypes.c_size_t
     L.matgptq_gemm.argtypes = [ci, ci, i64, i64, i64, vp, vp, vp, vp, vp, vp, u32]
     L.matgptq_gemm.restype = ci
+    L.matgptq_gemm_prologue.argtypes = [ci, ci, i64, i64, i64, vp, vp, vp, ci, vp, vp, vp, vp, ctypes.c_float, vp, vp, u32]
+    L.matgptq_gemm_prologue.restype = ci
     L.matgptq_pack_host.argtypes = [vp, i64, i64, ci, ci, vp]
     L.matgptq_pack_host.restype = ci
     L.matgptq_unpack_host.argtypes = [vp, i64, i64, ci, vp]

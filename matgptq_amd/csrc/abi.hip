@@ -27,6 +27,8 @@ int check_problem(int bits, int group_size, int64_t N, int64_t K);  // pack_host
   hipError_t launch_skinny_b##B(const GemmArgs&, int group_size, int r, int mb, bool master, hipStream_t);   \
   hipError_t launch_gemv_b##B(const GemmArgs&, int group_size, int shape, int W, size_t lds_pad, bool master, hipStream_t);  \
   hipError_t launch_gemv_b##B##_bf16(const GemmArgs&, int group_size, int shape, int W, size_t lds_pad, bool master, hipStream_t); \
+  hipError_t launch_gemv_prologue_b##B(const GemmArgs&, int kind, int shape, int W, const void* b, const void* w, void* out, \
+                                       float eps, hipStream_t);                                                            \
   hipError_t launch_skinny_b##B##_bf16(const GemmArgs&, int group_size, int r, int mb, bool master, hipStream_t); \
   hipError_t launch_decode_b##B##_bf16(const GemmArgs&, int group_size, int R, int S, int W,   \
                                        int kc, bool stream_flavour, size_t smem, hipStream_t); \
@@ -506,6 +508,7 @@ const char* matgptq_strerror(int code) {
     case MATGPTQ_EVARIANT: return "forced kernel variant does not apply to this problem";
     case MATGPTQ_ESIZE: return "size exceeds the supported maximum";
     case MATGPTQ_EWORKSPACE: return "workspace missing or smaller than matgptq_gemm_master_workspace_bytes()";
+    case MATGPTQ_EALIAS: return "an output buffer overlaps an input that other workgroups still read";
     case MATGPTQ_ESTATIC:
       return "the sliced tensor is larger than the library's built-in workspace (MATGPTQ_STATIC_WORKSPACE_BYTES): "
              "use matgptq_gemm_master with a workspace";
@@ -565,6 +568,61 @@ int matgptq_gemm(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
                  const void* x_dev, void* y_dev, void* stream, uint32_t flags) {
   return run_gemm(bitwidth, group_size, N, K, M, packed_dev, scales_dev, zeros_dev, x_dev, y_dev, stream,
                   flags, false);
+}
+
+int matgptq_gemm_prologue(int bitwidth, int group_size, int64_t N, int64_t K, int64_t M,
+                          const void* packed_dev, const void* scales_dev, const void* zeros_dev,
+                          int kind, const void* a_dev, const void* b_dev, const void* w_dev, void* out_dev,
+                          float eps, void* y_dev, void* stream, uint32_t flags) {
+  if (int e = check_problem(bitwidth, group_size, N, K)) return e;
+  if (M <= 0) return MATGPTQ_ESIZE;
+  if ((uint64_t)N * (uint64_t)K / 8 * (uint64_t)bitwidth >= (1ull << 32)) return MATGPTQ_ESIZE;
+  if (!packed_dev || !scales_dev || !a_dev || !y_dev) return MATGPTQ_ENULL;
+  if (kind != MATGPTQ_PRE_SILU_MUL && kind != MATGPTQ_PRE_ADD_RMSNORM) return MATGPTQ_EVARIANT;
+  if (group_size != 128 || (flags & MATGPTQ_FLAG_BF16) || M > kGemvMaxM || K % 128 != 0) return MATGPTQ_EVARIANT;
+  if (flags & (MATGPTQ_FLAG_VARIANT_MASK | MATGPTQ_FLAG_FLAVOUR_MASK)) return MATGPTQ_EVARIANT;
+  const int k_tiles = (int)(K / 128);
+  if (kind == MATGPTQ_PRE_ADD_RMSNORM) {
+    if (!w_dev) return MATGPTQ_ENULL;
+    if (k_tiles > 64) return MATGPTQ_EVARIANT;  // the mean needs all of K inside one round of a workgroup
+    const size_t row_bytes = (size_t)M * (size_t)K * 2;
+    auto overlaps = [&](const void* p) {
+      const char *o = static_cast<const char*>(out_dev), *q = static_cast<const char*>(p);
+      return p != nullptr && o < q + row_bytes && q < o + row_bytes;
+    };
+    if (out_dev && (overlaps(a_dev) || overlaps(b_dev))) return MATGPTQ_EALIAS;
+  }
+  Plan p;
+  if (int e = make_plan(bitwidth, group_size, N, K, M, zeros_dev != nullptr, flags, &p)) return e;
+  if (!p.gemv) return MATGPTQ_EVARIANT;
+  // the two shapes built with prologues: four tiles per wave, one or two row blocks per workgroup
+  const int shape = p.R >= 2 ? 2 : 1;
+  int W = (k_tiles + 3) / 4;
+  if (W > 16) W = 16;
+  GemmArgs a;
+  a.packed = static_cast<const uint32_t*>(packed_dev);
+  a.scales = static_cast<const uint16_t*>(scales_dev);
+  a.zeros = static_cast<const uint16_t*>(zeros_dev);
+  a.x = static_cast<const uint16_t*>(a_dev);
+  a.y = static_cast<uint16_t*>(y_dev);
+  a.N = (int)N;
+  a.K = (int)K;
+  a.M = (int)M;
+  a.G = (int)(K / group_size);
+  a.k_tiles = k_tiles;
+  a.row_blocks = (int)(N / 16);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t err;
+  switch (bitwidth) {
+    case 2: err = launch_gemv_prologue_b2(a, kind, shape, W, b_dev, w_dev, out_dev, eps, s); break;
+    case 3: err = launch_gemv_prologue_b3(a, kind, shape, W, b_dev, w_dev, out_dev, eps, s); break;
+    case 4: err = launch_gemv_prologue_b4(a, kind, shape, W, b_dev, w_dev, out_dev, eps, s); break;
+    case 6: err = launch_gemv_prologue_b6(a, kind, shape, W, b_dev, w_dev, out_dev, eps, s); break;
+    default: err = launch_gemv_prologue_b8(a, kind, shape, W, b_dev, w_dev, out_dev, eps, s); break;
+  }
+  if (err != hipSuccess) return MATGPTQ_ELAUNCH;
+  if (!(flags & MATGPTQ_FLAG_ASYNC) && hipStreamSynchronize(s) != hipSuccess) return MATGPTQ_ELAUNCH;
+  return MATGPTQ_OK;
 }
 
 // does the GEMM at this shape read the planes itself (gemv and mid-batch kernels), or does it need

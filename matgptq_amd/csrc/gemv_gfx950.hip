@@ -45,6 +45,14 @@ namespace {
 
 constexpr int kBits = MATGPTQ_BITS;
 
+constexpr int kPreNone = 0, kPreSiluMul = 1, kPreAddRmsNorm = 2;
+struct PrologueArgs {
+  const uint16_t* b;  // add + norm: the tensor added to the residual stream [M, K], or null
+  const uint16_t* w;  // add + norm: the norm's weight [K]
+  uint16_t* out;      // add + norm: where the new residual stream goes [M, K], or null
+  float eps;
+};
+
 __device__ __forceinline__ float dot2(half2v a, half2v b, float c) {
   return __builtin_amdgcn_fdot2(a, b, c, false);
 }
@@ -86,8 +94,18 @@ constexpr int gemv_lane_rows(int mb) { return mb < 4 ? mb : 4; }
 
 // MASTER: `a.packed` holds master-resident bit planes (master_layout.h); the rounded slice to
 // BITS is formed in registers while the raw pairs are built.
-template <int BITS, bool ZP, int GROUP, int T, int R, int MB, bool MASTER>
-__device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
+// PRE: the operator in front of the product is formed while the activations are staged, so that it
+// needs no launch and no round trip through memory of its own (group size 128, fp16 storage,
+// pre-sliced codes, up to four batch rows):
+//   kPreSiluMul     a.x is [M, 2 K]: x = fp16(silu(a.x[:, :K])) * a.x[:, K:], both roundings as two
+//                   element-wise operators make them;
+//   kPreAddRmsNorm  a.x is the residual stream h [M, K]: v = h + pro.b (one fp16 rounding; pro.b may be
+//                   null), x = fp16(v * rsqrt(mean(v^2) + eps) * pro.w), and the first workgroup writes v
+//                   to pro.out (another buffer than h: the other workgroups still read h).  The mean
+//                   needs every column, so the workgroup's one round must cover all of K.
+template <int BITS, bool ZP, int GROUP, int T, int R, int MB, bool MASTER, int PRE = kPreNone>
+__device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W, const PrologueArgs& pro) {
+  static_assert(PRE == kPreNone || (GROUP == 128 && !MASTER && MB <= 4 && !kBf16), "fused prologues: group 128, pre-sliced, fp16");
   using Fmt = TileFormat<BITS, MASTER>;
   constexpr bool kPerOctet = GROUP == 32;  // a scale per octet: the row groups of A take turns per octet
   static_assert(!kPerOctet || T <= 4, "one lane per 16 bytes of the zero block");
@@ -118,6 +136,7 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 
   unsigned char* xw = smem + wave * kWaveBytes;                   // this wave's X' and zeros
   float* red = reinterpret_cast<float*>(smem + W * kWaveBytes);   // [W][R * NV][64]
+  float* ssq_part = red + W * R * NV * 64;                        // add + norm: [W][MB] sums of squares
   if (lane * 16 < kZeroBytes) *reinterpret_cast<uint4*>(xw + kXBytes + lane * 16) = make_uint4(0, 0, 0, 0);
   float2* const osum = reinterpret_cast<float2*>(xw + kXBytes + kZeroBytes);  // group 32: [MB][T][4] (off, xs); eight batch rows: [MB][T]
 
@@ -146,13 +165,29 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
     // unconditional; what lies past the round is cut off by the size of its descriptor and
     // reads as zero (zero scale: such a tile adds nothing).
     u32x4 xv[MB][TH];
+    u32x4 xu[PRE == kPreNone ? 1 : MB][TH];  // second operand of the prologue (up half, or the added tensor)
+    u32x4 xn[TH];                            // add + norm: the norm's weights of these columns
 #pragma unroll
     for (int m = 0; m < MB; m++) {
       const int mrow = m < a.M ? m : a.M - 1;
-      const BufRsrc xr = make_rsrc(a.x + (size_t)mrow * a.K, (uint32_t)(kt0 + nt) * 256u);
+      const size_t row = (size_t)mrow * (PRE == kPreSiluMul ? 2 * (size_t)a.K : (size_t)a.K);
+      const BufRsrc xr = make_rsrc(a.x + row, (uint32_t)(kt0 + nt) * 256u);
 #pragma unroll
       for (int h = 0; h < TH; h++)
         xv[m][h] = __builtin_amdgcn_raw_buffer_load_b128(xr, lane * 16, (uint32_t)(kt0 + 4 * h) * 256u, 0);
+      if constexpr (PRE != kPreNone) {
+        const uint16_t* second = PRE == kPreSiluMul ? a.x + row + a.K : pro.b != nullptr ? pro.b + row : a.x;
+        const BufRsrc ur = make_rsrc(second, PRE == kPreAddRmsNorm && pro.b == nullptr ? 0u : (uint32_t)(kt0 + nt) * 256u);
+#pragma unroll
+        for (int h = 0; h < TH; h++)
+          xu[m][h] = __builtin_amdgcn_raw_buffer_load_b128(ur, lane * 16, (uint32_t)(kt0 + 4 * h) * 256u, 0);
+      }
+    }
+    if constexpr (PRE == kPreAddRmsNorm) {
+      const BufRsrc nr = make_rsrc(pro.w, (uint32_t)(kt0 + nt) * 256u);
+#pragma unroll
+      for (int h = 0; h < TH; h++)
+        xn[h] = __builtin_amdgcn_raw_buffer_load_b128(nr, lane * 16, (uint32_t)(kt0 + 4 * h) * 256u, 0);
     }
     uint16_t sv[R][NS], zv[R][NS];
     uint32_t w[R][T][Fmt::kWords];
@@ -191,6 +226,60 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
     // sums of every tile; after the rotate-reduce each lane of quarter q holds those of tile 4 h + q
     float off[MB][TH], xs[MB][TH];
     const half2v ones = h2_splat(1.0f);
+    if constexpr (PRE == kPreSiluMul) {
+#pragma unroll
+      for (int m = 0; m < MB; m++)
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          Frag g, u;
+          g.v = make_uint4(xv[m][h].x, xv[m][h].y, xv[m][h].z, xv[m][h].w);
+          u.v = make_uint4(xu[m][h].x, xu[m][h].y, xu[m][h].z, xu[m][h].w);
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            const float x = (float)g.h[e];
+            g.h[e] = (_Float16)(x / (1.0f + __expf(-x))) * u.h[e];
+          }
+          xv[m][h] = u32x4{g.u[0], g.u[1], g.u[2], g.u[3]};
+        }
+    } else if constexpr (PRE == kPreAddRmsNorm) {
+      float ssq[MB];
+#pragma unroll
+      for (int m = 0; m < MB; m++) {
+        ssq[m] = 0.f;
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          Frag v, d;
+          v.v = make_uint4(xv[m][h].x, xv[m][h].y, xv[m][h].z, xv[m][h].w);
+          d.v = make_uint4(xu[m][h].x, xu[m][h].y, xu[m][h].z, xu[m][h].w);  // zeros when nothing is added
+          v.h = v.h + d.h;
+          if (blockIdx.x == 0 && pro.out != nullptr && m < a.M && 4 * h + q < nt)
+            *reinterpret_cast<uint4*>(pro.out + (size_t)m * a.K + (size_t)(kt0 + 4 * h) * 128 + lane * 8) = v.v;
+#pragma unroll
+          for (int i = 0; i < 4; i++) ssq[m] = dot2(v.p[i], v.p[i], ssq[m]);
+          xv[m][h] = u32x4{v.u[0], v.u[1], v.u[2], v.u[3]};
+        }
+        float t = row_sum16(ssq[m]);
+        t += __shfl_xor(t, 16);
+        t += __shfl_xor(t, 32);
+        if (lane == 0) ssq_part[wave * MB + m] = t;
+      }
+      __syncthreads();  // every wave is here: the one round covers all of K (checked by the launcher)
+#pragma unroll
+      for (int m = 0; m < MB; m++) {
+        float total = 0.f;
+        for (int w2 = 0; w2 < W; w2++) total += ssq_part[w2 * MB + m];
+        const float rs = rsqrtf(total / (float)a.K + pro.eps);
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          Frag v, wn;
+          v.v = make_uint4(xv[m][h].x, xv[m][h].y, xv[m][h].z, xv[m][h].w);
+          wn.v = make_uint4(xn[h].x, xn[h].y, xn[h].z, xn[h].w);
+#pragma unroll
+          for (int e = 0; e < 8; e++) v.h[e] = (_Float16)((float)v.h[e] * rs * (float)wn.h[e]);
+          xv[m][h] = u32x4{v.u[0], v.u[1], v.u[2], v.u[3]};
+        }
+      }
+    }
 #pragma unroll
     for (int m = 0; m < MB; m++) {
 #pragma unroll
@@ -320,15 +409,18 @@ __device__ __forceinline__ void gemv_body(const GemmArgs& a, const int W) {
 }
 
 // WPE: waves per SIMD the register allocation is held to
-template <int BITS, bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER>
-__global__ void __launch_bounds__(1024, WPE) gemv_kernel(const GemmArgs a, const int W) {
-  gemv_body<BITS, ZP, GROUP, T, R, MB, MASTER>(a, W);
+template <int BITS, bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER, int PRE = kPreNone>
+__global__ void __launch_bounds__(1024, WPE) gemv_kernel(const GemmArgs a, const int W, const PrologueArgs pro) {
+  gemv_body<BITS, ZP, GROUP, T, R, MB, MASTER, PRE>(a, W, pro);
 }
 
-template <bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER>
-hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stream) {
+template <bool ZP, int GROUP, int T, int R, int MB, int WPE, bool MASTER, int PRE = kPreNone>
+hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stream, const PrologueArgs& pro = PrologueArgs{}) {
   const dim3 grid((a.row_blocks + R - 1) / R), block(64 * W);
-  size_t smem = (size_t)W * gemv_wave_lds(T, MB, GROUP) + (size_t)W * R * gemv_lane_rows(MB) * 256;
+  size_t smem = (size_t)W * gemv_wave_lds(T, MB, GROUP) + (size_t)W * R * gemv_lane_rows(MB) * 256 +
+                (PRE == kPreAddRmsNorm ? (size_t)W * MB * 4 : 0);
+  // add + norm: the workgroup's one round has to cover all of K, with every wave taking part
+  if (PRE == kPreAddRmsNorm && (W * T < a.k_tiles || (W - 1) * T >= a.k_tiles)) return hipErrorInvalidValue;
   if (smem < lds_pad) smem = lds_pad;
   if (W < 1 || W > 16 || a.M > MB || smem > 160 * 1024) return hipErrorInvalidValue;
   if (smem > 64 * 1024) {
@@ -339,14 +431,32 @@ hipError_t launch_one(const GemmArgs& a, int W, size_t lds_pad, hipStream_t stre
     if (const hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
     const uint64_t bit = 1ull << (dev & 63);
     if (dev >= 64 || !(allowed.load(std::memory_order_acquire) & bit)) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER>),
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER, PRE>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
       if (dev < 64) allowed.fetch_or(bit, std::memory_order_release);
     }
   }
-  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER>), grid, block, smem, stream, a, W);
+  hipLaunchKernelGGL((gemv_kernel<kBits, ZP, GROUP, T, R, MB, WPE, MASTER, PRE>), grid, block, smem, stream, a, W, pro);
   return hipGetLastError();
+}
+
+// the fused prologues: shapes (4, 1) and (4, 2), one, two or up to four batch rows
+template <bool ZP, int PRE>
+hipError_t launch_prologue(const GemmArgs& a, int shape, int W, const PrologueArgs& pro, hipStream_t s) {
+  if constexpr (kBf16) {
+    return hipErrorInvalidValue;
+  } else {
+    if (shape != 1 && shape != 2) return hipErrorInvalidValue;
+#define MATGPTQ_PRE_CASE(MBV)                                                                    \
+    return shape == 1 ? launch_one<ZP, 128, 4, 1, MBV, 4, false, PRE>(a, W, 0, s, pro)          \
+                      : launch_one<ZP, 128, 4, 2, MBV, 4, false, PRE>(a, W, 0, s, pro);
+    if (a.M == 1) { MATGPTQ_PRE_CASE(1) }
+    if (a.M == 2) { MATGPTQ_PRE_CASE(2) }
+    if (a.M <= 4) { MATGPTQ_PRE_CASE(4) }
+#undef MATGPTQ_PRE_CASE
+    return hipErrorInvalidValue;
+  }
 }
 
 // shapes built: (T tiles per wave and round, R row blocks per workgroup); the master-resident
@@ -403,6 +513,26 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 #else
 #define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(launch_gemv_b, MATGPTQ_BITS)
 #endif
+#if MATGPTQ_BF16
+#define MATGPTQ_PRE_LAUNCH_NAME MATGPTQ_CAT(MATGPTQ_CAT(launch_gemv_prologue_b, MATGPTQ_BITS), _bf16)
+#else
+#define MATGPTQ_PRE_LAUNCH_NAME MATGPTQ_CAT(launch_gemv_prologue_b, MATGPTQ_BITS)
+#endif
+// The gemv kernel with a fused prologue (kind 1: SiLU gate, 2: residual add + RMS norm); group size
+// 128, fp16 storage, up to four batch rows, shapes 1 and 2.
+hipError_t MATGPTQ_PRE_LAUNCH_NAME(const GemmArgs& a, int kind, int shape, int W, const void* b, const void* w,
+                                   void* out, float eps, hipStream_t stream) {
+  const PrologueArgs pro{static_cast<const uint16_t*>(b), static_cast<const uint16_t*>(w), static_cast<uint16_t*>(out), eps};
+  const bool zp = a.zeros != nullptr;
+  if (kind == kPreSiluMul)
+    return zp ? launch_prologue<true, kPreSiluMul>(a, shape, W, pro, stream)
+              : launch_prologue<false, kPreSiluMul>(a, shape, W, pro, stream);
+  if (kind == kPreAddRmsNorm)
+    return zp ? launch_prologue<true, kPreAddRmsNorm>(a, shape, W, pro, stream)
+              : launch_prologue<false, kPreAddRmsNorm>(a, shape, W, pro, stream);
+  return hipErrorInvalidValue;
+}
+
 hipError_t MATGPTQ_LAUNCH_NAME(const GemmArgs& a, int group_size, int shape, int W, size_t lds_pad, bool master,
                                hipStream_t stream) {
   if (group_size == 32)

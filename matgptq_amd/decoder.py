@@ -104,6 +104,7 @@ class Block(torch.nn.Module):
         self.cfg = cfg
         self.qkv, self.o = linears["qkv"], linears["o"]
         self.gate_up, self.down = linears["gate_up"], linears["down"]
+        self.fuse_prologues = True  # decode steps of up to four rows: norms and SiLU gate inside the linears
         self.input_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=dtype, device=device), requires_grad=False)
         self.post_norm = torch.nn.Parameter(torch.ones(cfg.hidden, dtype=dtype, device=device), requires_grad=False)
 
@@ -131,18 +132,26 @@ class Block(torch.nn.Module):
         return h
 
     def forward_fused(self, h, delta, x, cos_table, sin_table, pos, k_cache, v_cache, attn_workspace):
-        """The same block for a few rows with the operators between the linears fused (nine
-        launches): `h` [M, hidden] is updated in place with `delta` (the previous block's last
-        linear output, or None) and this block's attention output; returns the output of `down`,
-        which the next block (or the final norm) adds.  `x` [M, hidden] is scratch,
-        `attn_workspace` the workspace of the split attention or None for the unsplit one.  Eight
-        launches for a single row (nine with the split attention)."""
+        """The same block for a few rows with the operators between the linears fused: `h` [M, hidden]
+        is updated in place with `delta` (the previous block's last linear output, or None) and this
+        block's attention output; returns the output of `down`, which the next block (or the final
+        norm) adds.  `x` [M, hidden] is scratch, `attn_workspace` the workspace of the split attention
+        or None for the unsplit one.  Five launches for a single row (six with the split attention),
+        eight or nine where the linears cannot take their prologues in the kernel."""
         from . import _glue
+        from .ops import PRE_ADD_RMSNORM, PRE_SILU_MUL
 
         cfg = self.cfg
         m = h.shape[0]
-        _glue.add_rmsnorm(h, delta, self.input_norm, x, cfg.rms_eps)
-        qkv = self.qkv(x)
+        # Up to four rows the two norms and the SiLU gate ride in the linears behind them (five launches
+        # per block instead of eight): the residual stream goes h -> x (= h + delta) in the qkv launch
+        # and x -> h (= x + attention output) in the gate_up launch, so it is back in `h` at the end.
+        in_kernel = self.prologues_apply(m)
+        if in_kernel:
+            qkv = self.qkv.forward_prologue(PRE_ADD_RMSNORM, h, delta, self.input_norm, x, cfg.rms_eps)
+        else:
+            _glue.add_rmsnorm(h, delta, self.input_norm, x, cfg.rms_eps)
+            qkv = self.qkv(x)
         attn = torch.empty(m, cfg.hidden, dtype=h.dtype, device=h.device)
         # For a single row the rotary embedding and the cache write ride in the attention launch.
         # A long cache is split over workgroups (two launches; measured on MI355X with 32 / 8 heads,
@@ -156,10 +165,29 @@ class Block(torch.nn.Module):
             _glue.rope_attention(qkv, cos_table, sin_table, pos, k_cache, v_cache, attn, cfg.heads, cfg.kv_heads)
         else:
             _glue.attention(qkv, k_cache, v_cache, pos, attn, cfg.heads, cfg.kv_heads)
+        if in_kernel:
+            gate_up = self.gate_up.forward_prologue(PRE_ADD_RMSNORM, x, self.o(attn), self.post_norm, h, cfg.rms_eps)
+            return self.down.forward_prologue(PRE_SILU_MUL, gate_up)
         _glue.add_rmsnorm(h, self.o(attn), self.post_norm, x, cfg.rms_eps)
         act = torch.empty(m, cfg.ffn, dtype=h.dtype, device=h.device)
         _glue.silu_mul(self.gate_up(x), act)
         return self.down(act)
+
+    def prologues_apply(self, rows: int) -> bool:
+        """Whether this block's qkv, gate_up and down linears take their prologues in the kernel."""
+        from .ops import PRE_ADD_RMSNORM, PRE_SILU_MUL, prologue_applies
+
+        if not self.fuse_prologues:
+            return False
+        cfg, dtype = self.cfg, self.input_norm.dtype
+        def plain(lin):  # a pre-sliced layer without act-order permutation, as a module or behind the plugin
+            params = getattr(lin, "layer", lin)
+            return (hasattr(lin, "forward_prologue") and getattr(params, "matgptq_perm", None) is None
+                    and getattr(params, "matgptq_planes", None) is None)
+
+        return (all(plain(lin) for lin in (self.qkv, self.gate_up, self.down))
+                and prologue_applies(PRE_ADD_RMSNORM, rows, cfg.hidden, cfg.group_size, dtype)
+                and prologue_applies(PRE_SILU_MUL, rows, cfg.ffn, cfg.group_size, dtype))
 
 
 def _rotate(t, cos, sin):
@@ -253,6 +281,9 @@ class PluginLinear(torch.nn.Module):
 
     def forward(self, x):
         return self.method.apply(self.layer, x)
+
+    def forward_prologue(self, kind, a, added=None, norm_weight=None, residual_out=None, eps=1e-5):
+        return self.method.apply_prologue(self.layer, kind, a, added, norm_weight, residual_out, eps)
 
 
 def random_mixnmatch_decoder(cfg: DecoderConfig, max_context: int, bit_choices: Sequence[int] = (2, 3, 4, 6, 8),

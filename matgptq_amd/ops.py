@@ -22,6 +22,11 @@ Additive operators of this implementation (all under torch.ops.matgptq_cuda):
     matmul_matgptq_master           matmul_matgptq_zp on those planes with `bitwidth` as a run-time
                                     argument: the rounded slice is formed in registers
     unpack_matgptq_master_resident  planes -> the uint8 codes the GEMM sees at `bitwidth`
+
+and, as a plain function over the C ABI (not a registered operator):
+
+    matmul_matgptq_prologue  the decode product with the operator in front of it fused into the kernel
+                             (SiLU gate of a fused gate_up output, or residual add + RMS norm)
 """
 from __future__ import annotations
 
@@ -99,3 +104,48 @@ def matryoshka_slice(x: torch.Tensor, master_bitwidth: int, slice_bitwidth: int)
     if master_bitwidth == slice_bitwidth:
         return floor.clamp_(0, top).to(torch.uint8)
     return (floor + ((v >> (drop - 1)) & 1)).clamp_(0, top).to(torch.uint8)
+
+
+PRE_SILU_MUL, PRE_ADD_RMSNORM = 1, 2
+
+
+def prologue_applies(kind: int, rows: int, n_in_features: int, group_size: int, dtype: torch.dtype) -> bool:
+    """Whether `matmul_matgptq_prologue` covers this call (include/matgptq_abi.h: fp16 storage,
+    group size 128, up to four rows; the norm needs all of K inside one round: K <= 8192)."""
+    return (dtype == torch.float16 and group_size == 128 and 1 <= rows <= 4 and n_in_features % 128 == 0
+            and (kind == PRE_SILU_MUL or (kind == PRE_ADD_RMSNORM and n_in_features <= 8192)))
+
+
+def matmul_matgptq_prologue(kind: int, a: torch.Tensor, matgptq_weights: torch.Tensor, matgptq_scales: torch.Tensor,
+                            matgptq_zeros, n_out_features: int, n_in_features: int, bitwidth: int, group_size: int,
+                            added=None, norm_weight=None, residual_out=None, eps: float = 1e-5) -> torch.Tensor:
+    """`matmul_matgptq[_zp]` on activations the kernel forms itself while staging them:
+
+    PRE_SILU_MUL     a [M, 2K] = (gate | up)  ->  x = silu(gate) * up
+    PRE_ADD_RMSNORM  a [M, K] the residual stream; v = a + added (added may be None), x = rms_norm(v) *
+                     norm_weight; v is written to `residual_out` (not a or `added`) when given
+
+    Launches on the current stream, allocates only the output; raises where the fused kernel does not
+    apply (see `prologue_applies`)."""
+    from . import _lib
+
+    rows = a.shape[0]
+    for t in (a, added, norm_weight, residual_out):
+        if t is not None and (t.dtype != torch.float16 or not t.is_cuda or not t.is_contiguous()):
+            raise ValueError("matmul_matgptq_prologue: contiguous float16 tensors on the GPU expected")
+    width = 2 * n_in_features if kind == PRE_SILU_MUL else n_in_features
+    if a.dim() != 2 or a.shape[1] != width:
+        raise ValueError("matmul_matgptq_prologue: input has the wrong shape")
+    for t in (added, residual_out):
+        if t is not None and t.shape != a.shape:
+            raise ValueError("matmul_matgptq_prologue: added tensor and residual output take the input's shape")
+    if kind == PRE_ADD_RMSNORM and (norm_weight is None or norm_weight.numel() != n_in_features):
+        raise ValueError("matmul_matgptq_prologue: the norm needs a weight of n_in_features elements")
+    y = torch.empty((rows, n_out_features), dtype=torch.float16, device=a.device)
+    ptr = lambda t: None if t is None else t.data_ptr()
+    with torch.cuda.device(a.device):
+        _lib.check(_lib.load().matgptq_gemm_prologue(
+            bitwidth, group_size, n_out_features, n_in_features, rows, matgptq_weights.data_ptr(),
+            matgptq_scales.data_ptr(), ptr(matgptq_zeros), kind, a.data_ptr(), ptr(added), ptr(norm_weight),
+            ptr(residual_out), eps, y.data_ptr(), torch.cuda.current_stream().cuda_stream, 1))
+    return y

@@ -71,3 +71,17 @@ class MatGPTQLinear(torch.nn.Module):
         return torch.ops.matgptq_cuda.matmul_matgptq(
             x, self.matgptq_qweight, self.matgptq_scales,
             self.n_out_features, self.n_in_features, self.bitwidth, self.group_size, self.flag)
+
+    @torch.no_grad()
+    def forward_prologue(self, kind: int, a: torch.Tensor, added=None, norm_weight=None, residual_out=None,
+                         eps: float = 1e-5) -> torch.Tensor:
+        """Additive: `forward` on activations that the kernel forms while it stages them (the SiLU gate
+        of a fused gate_up output, or residual add + RMS norm; `matgptq_amd.ops.matmul_matgptq_prologue`).
+        Up to four rows, fp16, group size 128, no act-order permutation."""
+        from matgptq_amd import ops
+
+        if self.matgptq_perm is not None:
+            raise RuntimeError("the fused prologues do not apply to a layer with an act-order permutation")
+        return ops.matmul_matgptq_prologue(kind, a, self.matgptq_qweight, self.matgptq_scales, self.matgptq_zeros,
+                                           self.n_out_features, self.n_in_features, self.bitwidth, self.group_size,
+                                           added, norm_weight, residual_out, eps)

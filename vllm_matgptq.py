@@ -330,3 +330,19 @@ class MatGPTQLinearMethod(LinearMethodBase):
         if bias is not None:
             y += bias
         return y
+
+    def apply_prologue(self, layer: torch.nn.Module, kind: int, a: torch.Tensor, added=None, norm_weight=None,
+                       residual_out=None, eps: float = 1e-5) -> torch.Tensor:
+        """Additive (no counterpart in the reference): `apply` for decode steps of up to four rows with
+        the operator in front of the linear formed inside the kernel - `kind` 1: `a` is the fused
+        gate_up output [M, 2K], x = silu(gate) * up; 2: `a` is the residual stream, x = rms_norm(a +
+        added) * norm_weight, a + added written to `residual_out`.  Pre-sliced fp16 layers at group
+        size 128 without act-order; callers check `matgptq_amd.ops.prologue_applies` first."""
+        from matgptq_amd import ops
+
+        if getattr(layer, "matgptq_perm", None) is not None or getattr(layer, "matgptq_planes", None) is not None:
+            raise RuntimeError("the fused prologues take pre-sliced layers without an act-order permutation")
+        return ops.matmul_matgptq_prologue(kind, a, layer.matgptq_weights, layer.matgptq_scales,
+                                           getattr(layer, "matgptq_zeros", None), self.n_out_features,
+                                           self.n_in_features, getattr(layer, "matgptq_bitwidth", self.bitwidth),
+                                           self.config.group_size, added, norm_weight, residual_out, eps)
