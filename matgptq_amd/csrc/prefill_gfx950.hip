@@ -39,6 +39,9 @@
 // those rows in their L2; the ring tile keeps the plain order.
 #include "device_common.h"
 
+// (m0 in the clobber list of the LDS copies below: reserved, but the compiler keeps nothing in it)
+#pragma clang diagnostic ignored "-Winline-asm"
+
 #ifndef MATGPTQ_BITS
 #error "compile with -DMATGPTQ_BITS={2,3,4,6,8}"
 #endif
@@ -117,8 +120,8 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile offsets stay scalar
-  const int wave = KS == 1 && !PAIR ? wave_wg : (wave_wg & 3);  // within its group of four
-  const int grp = KS == 1 && !PAIR ? 0 : (wave_wg >> 2);
+  const int wave = wave_wg & 3;  // within its group of four
+  const int grp = KS == 1 && !PAIR ? 0 : ((wave_wg >> 2) & 1);
   if constexpr (PAIR) lid = 2 * lid + grp;
   // K tiles [k_lo, k_hi) in kt_n trips (the same count for both groups: they share the barriers; a
   // tile beyond k_hi reads as zeros)
@@ -297,11 +300,32 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       const int ih = step + 2 * k_lo;
       const bool valid = ih < 2 * k_hi;
       const BufRsrc xres = make_rsrc(a.x, valid ? x_bytes : 0u);
+      if constexpr (KS == 2 || PAIR) {
+        // Workgroups of eight waves issue the copies as assembly text.  The compiler places its own
+        // counter waits in front of LDS reads that may overlap a copy in flight and, on loop paths that
+        // are never taken, in front of the first use of the weights; it cannot tell the ring buffers
+        // apart, so these waits let nothing stay in flight.  A wave that stalls there holds up both
+        // groups at the next barrier.  Copies it does not see leave only the hand-counted waits, which
+        // every LDS read of copied data already sits behind; its own waits for register loads count
+        // fewer loads than are in flight and stay on the safe side.  (Measured at 4 bits: 6 to 10 %
+        // faster where K is split in the workgroup, no difference in workgroups of four waves, which
+        // keep the intrinsic.)
+        const uint64_t xa = (uint64_t)(uintptr_t)a.x;
+        const u32x4 xd = {(uint32_t)xa, (uint32_t)(xa >> 32) & 0xffffu, valid ? x_bytes : 0u, 0x00020000u};
+        const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(ring + wave * 32 * kXs);
 #pragma unroll
-      for (int i = 0; i < 4; i++)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            xres, (__attribute__((address_space(3))) void*)(ring + (wave * 32 + i * 8) * kXs), 16, dma_voff[i],
-            (uint32_t)ih * (kXs * 2), 0, 0);
+        for (int i = 0; i < 4; i++)  // m0: LDS address of the wave's 8 rows; one wait state before its use
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                       :
+                       : "s"(base + i * 8 * kXs * 2), "v"(dma_voff[i]), "s"(xd), "s"((uint32_t)ih * (kXs * 2))
+                       : "memory", "m0");
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              xres, (__attribute__((address_space(3))) void*)(ring + (wave * 32 + i * 8) * kXs), 16, dma_voff[i],
+              (uint32_t)ih * (kXs * 2), 0, 0);
+      }
     };
     // operand read: row i*16 + r16, columns [jj*32 + q*8, +8)
     const int sw = (r16 >> 1) & 7;
@@ -325,6 +349,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     // matrix work, which is why a single operand set is enough.
     Frag aw[RBW];
     Frag bv[MT];
+    constexpr bool kReloadBehindBranch = GROUP != 32;  // see the loops below
     auto dstep = [&](const uint32_t (&w)[RBW][BITS], const uint32_t (&sv)[RBW][GPT], const uint32_t (&zv)[RBW][GPT],
                      auto jtag, const _Float16* nring, int njj) {
       dequant_step(aw, w, sv, zv, jtag);
@@ -446,11 +471,16 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
         dma(rb, 2 * kb + 5);
         dstep(wcur, sc, zc, J3{}, rn, 0);
         refill(J3{}, kb + 1);
-        load_aux(sc, zc, kb + 2);  // this set is free now
       };
+      // (S(t+2), into the set that tile t has just left, is issued behind the branch: see the loop below)
       for (int kb = 0; kb < kt_n; kb += 2) {
         stile(kb, scur, zcur, ring0, ring1, ring2);
-        if (kb + 1 < kt_n) stile(kb + 1, snxt, znxt, ring2, ring3, ring0);
+        if constexpr (!kReloadBehindBranch) load_aux(scur, zcur, kb + 2);
+        if (kb + 1 < kt_n) {
+          if constexpr (kReloadBehindBranch) load_aux(scur, zcur, kb + 2);
+          stile(kb + 1, snxt, znxt, ring2, ring3, ring0);
+          load_aux(snxt, znxt, kb + 3);
+        }
       }
     } else {
     // buffer loads one load_weights() issues: the codes, then a scale (and a zero) per group
@@ -482,11 +512,23 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
         wait_and_meet(std::integral_constant<int, 8 + kW>{});
         dma(rb, 2 * kb + 5);
         dstep(wc, sc, zc, J3{}, rn, 0);
-        load_weights(wc, sc, zc, kb + 2);  // this set is free now
       };
+      // W(t+2) goes into the set that tile t has just left.  The first tile's set is reloaded behind
+      // the branch, not in front of it: the compiler places its own counter waits over every path of
+      // the flow graph, and the path that skips the second tile leads from the end of the first
+      // straight back to its start.  With the reload in front of the branch, the loads the top of the
+      // loop needs would be the youngest ones on that path, and its waits would let nothing stay in
+      // flight; on the path that is taken, a whole tile's loads are younger.  (Group size 32 keeps the
+      // reload in front: with four scales and zeros per row block the registers are full, and the
+      // other order spills.)
       for (int kb = 0; kb < kt_n; kb += 2) {
         dtile(kb, wcur, scur, zcur, ring0, ring1, ring2);
-        if (kb + 1 < kt_n) dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
+        if constexpr (!kReloadBehindBranch) load_weights(wcur, scur, zcur, kb + 2);
+        if (kb + 1 < kt_n) {
+          if constexpr (kReloadBehindBranch) load_weights(wcur, scur, zcur, kb + 2);
+          dtile(kb + 1, wnxt, snxt, znxt, ring2, ring3, ring0);
+          load_weights(wnxt, snxt, znxt, kb + 3);
+        }
       }
     }
   } else {
