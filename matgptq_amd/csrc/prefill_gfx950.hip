@@ -300,16 +300,16 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       const int ih = step + 2 * k_lo;
       const bool valid = ih < 2 * k_hi;
       const BufRsrc xres = make_rsrc(a.x, valid ? x_bytes : 0u);
-      if constexpr (KS == 2 || PAIR) {
-        // Workgroups of eight waves issue the copies as assembly text.  The compiler places its own
+      if constexpr (KS == 2 && RBW < 4) {
+        // The narrower tiles with K split in the workgroup issue the copies as assembly text.  The compiler places its own
         // counter waits in front of LDS reads that may overlap a copy in flight and, on loop paths that
         // are never taken, in front of the first use of the weights; it cannot tell the ring buffers
         // apart, so these waits let nothing stay in flight.  A wave that stalls there holds up both
         // groups at the next barrier.  Copies it does not see leave only the hand-counted waits, which
         // every LDS read of copied data already sits behind; its own waits for register loads count
-        // fewer loads than are in flight and stay on the safe side.  (Measured at 4 bits: 6 to 10 %
-        // faster where K is split in the workgroup, no difference in workgroups of four waves, which
-        // keep the intrinsic.)
+        // fewer loads than are in flight and stay on the safe side.  (Measured at 4 bits: 128 x 128 and
+        // 128 x 192 tiles with K split 2 to 10 % faster; the 128 x 256 tile 1 to 2 % slower with K split,
+        // no difference in pairs or in workgroups of four waves: those keep the intrinsic.)
         const uint64_t xa = (uint64_t)(uintptr_t)a.x;
         const u32x4 xd = {(uint32_t)xa, (uint32_t)(xa >> 32) & 0xffffu, valid ? x_bytes : 0u, 0x00020000u};
         const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(ring + wave * 32 * kXs);
