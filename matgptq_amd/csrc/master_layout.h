@@ -32,6 +32,14 @@ namespace matgptq {
 
 constexpr int kMasterTileWords = 512;
 
+// full unrolling of the small loops below in device code: left rolled, the word a plane's bits go to
+// is picked by a chain of compares and selects per code
+#if defined(__clang__)
+#define MATGPTQ_UNROLL _Pragma("unroll")
+#else
+#define MATGPTQ_UNROLL
+#endif
+
 // words a lane reads at bitwidth b
 constexpr int master_words(int b) { return b == 2 ? 3 : b == 3 ? 4 : b == 4 ? 5 : 8; }
 
@@ -46,7 +54,9 @@ MATGPTQ_HD int master_word_offset(int lane, int w) {
 // the lane's 32 master codes (index j*8 + e) -> its eight words
 MATGPTQ_HD void master_encode_lane(const uint8_t (&codes)[32], uint32_t (&w)[8]) {
   for (int i = 0; i < 8; i++) w[i] = 0;
+  MATGPTQ_UNROLL
   for (int j = 0; j < 4; j++)
+    MATGPTQ_UNROLL
     for (int e = 0; e < 8; e++) {
       const uint32_t c = codes[j * 8 + e];
       const int nb = nibble_of(e), d = j >> 1, u = j & 1;
@@ -116,6 +126,7 @@ MATGPTQ_HD uint8_t master_code(const uint32_t* w, int e) {
 // all 32 sliced codes of a lane (index j*8 + e)
 template <int BITS>
 MATGPTQ_HD void master_decode_lane(const uint32_t* w, uint8_t (&codes)[32]) {
+  MATGPTQ_UNROLL
   for (int e = 0; e < 8; e++) {
     codes[e] = master_code<BITS, 0>(w, e);
     codes[8 + e] = master_code<BITS, 1>(w, e);
