@@ -473,8 +473,8 @@ def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
     # The prefill and mid-batch kernels multiply bf16 by bf16 on the matrix cores.  With the identity as
     # activations every output is one weight (plus exact zeros), so the result must be
     # dequantize() on bfloat16 tensors, bit for bit (integer zero points: one rounding on both
-    # sides).  Ring tiles 128 x 256, 128 x 128, 128 x 192, the tail split, a staged tile, the two
-    # tiles that split K inside the workgroup, and three shapes of the mid-batch kernel.
+    # sides).  Ring tiles 128 x 256, 128 x 128, 128 x 192, the tail split, a staged tile, the three
+    # tiles that split K inside the workgroup, the paired tiles, and three shapes of the mid-batch kernel.
     n, k, g = 304, 256, 128
     q, s16, z16 = o.make_layer(n, k, g, seed=300 + b, symmetric=not zp)
     s = o.round_to_bf16(s16.astype(np.float32))
@@ -482,7 +482,7 @@ def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
     x = np.eye(k, dtype=np.float32)
     pk = G.pack_device(q, b, True)
     w = o.dequantize_bf16(q, s, z, b, g)
-    for cfg in (64, 67, 73, 72, 66, 74, 75, 80, 84, 88):
+    for cfg in (64, 67, 73, 72, 66, 74, 75, 76, 77, 80, 84, 88):
         y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | (cfg << 8))
         assert np.array_equal(y, w.T), (b, zp, cfg)
 
