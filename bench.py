@@ -17,8 +17,8 @@ The JSON line also carries
   cpu_baseline the reference's PyTorch CPU path (slice -> dequantize -> F.linear,
                restated in oracle/torch_path.py) on the host cores, same layers, one pass
   summary      a dozen scalars of the tables below
-The per-bitwidth / per-layer / small-batch / M=2048 prefill tables go to gpurun_out/bench_extra.json
-and to stderr, one table per line; the last stdout line stays under 4 KB.
+The per-bitwidth / per-layer / small-batch / M=2048 prefill tables go to a side file (EXTRA_FILE,
+named in the line's `tables` key) and to stderr, one table per line; the last stdout line stays under 4 KB.
 """
 from __future__ import annotations
 
