@@ -10,6 +10,7 @@
 
 #include "../../include/matgptq_abi.h"
 #include "device_common.h"
+#include "prefill_plan.h"
 
 // Scratch of matgptq_gemm_master_static: device memory that lives in the library's code object, so
 // that entry point needs no allocation at all.  One copy per GPU, at its own address.
@@ -211,6 +212,11 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         // second round starts and the 128 x 256 tile is ahead again (6144 x 4096, M = 2560: 139
         // against 108 us).
         p->cfg = 9;
+        // ... and where those leave slots empty while 128 x 128 tiles would need a second round, both
+        // widths in one launch take every slot once (10240 x 8192 at M = 1024: 432 tiles of 192 rows on
+        // 512 slots; 256 of them and 256 of 128 rows instead)
+        int narrow = 0;
+        if (prefill_mix_wide_tiles(row_blocks, m_tiles, &narrow) > 0) p->cfg = 14;
       }
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
@@ -378,7 +384,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       R = 1 << ((variant - 80) % 3);
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
-      if (variant - 64 > 13) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 14) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 64;

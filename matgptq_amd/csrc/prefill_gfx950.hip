@@ -38,6 +38,7 @@
 // congruent modulo 8) walk consecutive activation tiles of the same weight rows and share
 // those rows in their L2; the ring tile keeps the plain order.
 #include "device_common.h"
+#include "prefill_plan.h"
 
 // (m0 in the clobber list of the LDS copies below: reserved, but the compiler keeps nothing in it)
 #pragma clang diagnostic ignored "-Winline-asm"
@@ -761,6 +762,34 @@ prefill_tail8_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
     prefill_body<BITS, GROUP, ZP, 2, 8, 2>(a, blockIdx.x - n_pairs, m_tiles, rb_tail, lds);
 }
 
+// Two tile widths sized to fill the resident slots in one round (prefill_mix_wide_tiles): the first
+// `n_big` workgroups take 128 x 192 tiles of the weight rows below row block `rb_tail`, the others
+// 128 x 128 tiles of the rest.  Workgroups are placed in the order of their ids, the least loaded CU
+// first, so a CU ends up with one of each.
+template <int BITS, int GROUP, bool ZP>
+__global__ void __launch_bounds__(256, 2)
+prefill_mix_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
+  static_assert(prefill_lds_halves(3, 8) == prefill_lds_halves(2, 8), "both tiles share one LDS block");
+  __shared__ __align__(16) _Float16 lds[prefill_lds_halves(3, 8)];
+  if ((int)blockIdx.x < n_big)
+    prefill_body<BITS, GROUP, ZP, 3, 8>(a, blockIdx.x, m_tiles, 0, lds);
+  else
+    prefill_body<BITS, GROUP, ZP, 2, 8>(a, blockIdx.x - n_big, m_tiles, rb_tail, lds);
+}
+
+template <int GROUP, bool ZP>
+hipError_t launch_mix(const GemmArgs& a, hipStream_t stream) {
+  const int m_tiles = (a.M + 127) / 128;
+  int narrow = 0;
+  const int wide = prefill_mix_wide_tiles(a.row_blocks, m_tiles, &narrow);
+  // (forced on a shape the mix does not apply to: narrow tiles only)
+  const int rb_tail = wide * 12;
+  const int n_small = wide > 0 ? narrow : (a.row_blocks + 7) / 8;
+  const dim3 grid((wide + n_small) * m_tiles), block(256);
+  hipLaunchKernelGGL((prefill_mix_kernel<kBits, GROUP, ZP>), grid, block, 0, stream, a, m_tiles, wide * m_tiles, rb_tail);
+  return hipGetLastError();
+}
+
 template <int GROUP, bool ZP>
 hipError_t launch_tail8(const GemmArgs& a, hipStream_t stream) {
   const int m_tiles = (a.M + 127) / 128;
@@ -824,6 +853,7 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 9: return launch_cfg<GROUP, ZP, 3, 8>(a, s);   // 128 x 192
     case 12: return launch_tail8<GROUP, ZP>(a, s);      // 128 x 256 in pairs, then a tail of 128 x 128 with K split
     case 13: return launch_split<GROUP, ZP, 3, 8>(a, s);  // 128 x 192, K split in the workgroup
+    case 14: return launch_mix<GROUP, ZP>(a, s);          // 128 x 192 and 128 x 128, one round of all slots
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 #endif

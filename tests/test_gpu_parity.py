@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(14))
+@pytest.mark.parametrize("cfg", range(15))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -324,6 +324,45 @@ def test_prefill_paired_tiles_with_a_split_tail_odd_tile_count(zp):
     y8 = lay.run(x, flags=1 | ((64 + 8) << 8))
     assert np.array_equal(y[:, :1792], y8[:, :1792])
     assert np.max(np.abs(y[:, 1792:].astype(np.float64) - y8[:, 1792:])) <= 2e-3 * np.max(np.abs(y8.astype(np.float64)))
+
+
+@pytest.mark.parametrize("b,g,zp", ((4, 128, True), (4, 128, False), (2, 128, True), (3, 128, True), (8, 128, True),
+                                    (6, 128, True), (4, -1, True), (4, 32, False)))
+def test_prefill_two_tile_widths_in_one_launch(b, g, zp):
+    # 65 row blocks, 73 activation tiles (7 slots per column): 3 tiles of 192 rows take the first 36 row
+    # blocks, 4 tiles of 128 rows the other 29 (the last one ragged); ragged M.  Both parts run the
+    # arithmetic of their own tile, so each equals the launch that uses that width alone.
+    n, k, m = 1040, 384, 73 * 128 - 5
+    lay = G.Layer(n, k, b, g, seed=14 + b, zero_points=zp)
+    x = o.make_activations(m, k, seed=14)
+    assert _lib.describe_plan(b, g, n, k, m, zp, 1 | ((64 + 14) << 8)).endswith("cfg14")
+    y = lay.run(x, flags=1 | ((64 + 14) << 8))
+    G.assert_close_to_oracle(y, x, lay.w, f"two widths b={b} g={g} zp={zp}")
+    G.assert_regression_bound(y, x, lay.w, f"two widths b={b} g={g} zp={zp}")
+    wide = lay.run(x, flags=1 | ((64 + 9) << 8))
+    narrow = lay.run(x, flags=1 | ((64 + 3) << 8))
+    assert np.array_equal(y[:, :576], wide[:, :576])
+    assert np.array_equal(y[:, 576:], narrow[:, 576:])
+
+
+def test_prefill_two_tile_widths_forced_where_they_do_not_apply():
+    # one round of narrow tiles is enough here: the launch degenerates to those
+    n, k, m = 304, 128 * 7, 200
+    lay = G.Layer(n, k, 4, 128, seed=3)
+    x = o.make_activations(m, k, seed=3)
+    y = lay.run(x, flags=1 | ((64 + 14) << 8))
+    assert np.array_equal(y, lay.run(x, flags=1 | ((64 + 3) << 8)))
+
+
+def test_llama3_70b_qkv_at_1024_rows_takes_both_widths():
+    n, k, m = 10240, 8192, 1024
+    assert _lib.describe_plan(4, 128, n, k, m, True).endswith("cfg14")
+    lay = G.Layer(n, k, 4, 128, seed=1)
+    x = o.make_activations(m, k, seed=1)
+    y = lay.run(x)
+    assert np.all(np.isfinite(y))
+    rows = np.array([0, 129, 1023])
+    G.assert_close_to_oracle(y[rows], x[rows], lay.w, "70B qkv at M = 1024")
 
 
 def test_llama3_70b_qkv_prefill_full_size_with_tail_tiles():

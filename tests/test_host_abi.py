@@ -237,9 +237,24 @@ def test_planner_takes_192_row_tiles_where_they_fill_one_round_better():
     for bits in (2, 3, 4, 8):
         assert _lib.describe_plan(bits, 128, 6144, 4096, 2048, True).endswith("cfg9")
     assert _lib.describe_plan(4, 32, 6144, 4096, 2048, False).endswith("cfg9")
-    assert _lib.describe_plan(4, -1, 5120, 4096, 2048, True).endswith("cfg9")
     assert _lib.describe_plan(4, 128, 6144, 4096, 2560, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 7168, 4096, 2048, True).endswith("cfg0")
+
+
+def test_planner_mixes_two_tile_widths_where_neither_fills_the_one_round():
+    # 5120 rows at M = 2048: 32 slots per column of activation tiles; 27 tiles of 192 rows leave five
+    # empty, 40 of 128 rows need a second round: 16 of 192 and 16 of 128 take every slot once
+    assert _lib.describe_plan(4, -1, 5120, 4096, 2048, True).endswith("cfg14")
+    for bits in (2, 3, 4, 8):
+        assert _lib.describe_plan(bits, 128, 10240, 8192, 1024, True).endswith("cfg14")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 1024, False).endswith("cfg14")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 1024, True, 3).endswith("cfg14")  # bf16 storage at 4 bits
+    # formats that do not take the 128 x 192 tile in that regime keep their own choice
+    assert not _lib.describe_plan(6, 128, 10240, 8192, 1024, True).endswith("cfg14")
+    assert not _lib.describe_plan(4, 32, 10240, 8192, 1024, True).endswith("cfg14")
+    # exactly one round of 128 x 192 tiles, or of 128 x 128 tiles: no mix
+    assert _lib.describe_plan(4, 128, 6144, 4096, 2048, True).endswith("cfg9")
+    assert not _lib.describe_plan(4, 128, 8192, 8192, 1024, True).endswith("cfg14")
 
 
 def test_planner_splits_k_in_the_workgroup_where_ring_tiles_would_sit_one_per_cu():
@@ -284,7 +299,7 @@ def test_planner_gives_bf16_storage_the_wide_ring_tile_where_its_registers_hold(
             assert _lib.describe_plan(bits, 128, 10240, 8192, 2048, zp, 3) == _lib.describe_plan(bits, 128, 10240, 8192, 2048, zp, 1)
             assert _lib.describe_plan(bits, 128, 57344, 8192, 2048, zp, 3).endswith("cfg0")
             assert _lib.describe_plan(bits, -1, 8192, 28672, 2048, zp, 3).endswith("cfg0")
-    assert _lib.describe_plan(4, 128, 10240, 8192, 1024, True, 3).endswith("cfg9")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 1024, True, 3).endswith("cfg14")  # (both widths in one launch)
     assert _lib.describe_plan(8, -1, 8192, 8192, 2048, True, 3).endswith("cfg0")
     assert _lib.describe_plan(4, 32, 8192, 8192, 2048, False, 3).endswith("cfg3")
     assert _lib.describe_plan(3, 128, 8192, 8192, 2048, True, 3).endswith("cfg3")
