@@ -162,6 +162,15 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       // that the last part of the launch runs two waves per SIMD as well (10240 x 8192 at M = 2048:
       // 285 -> 276 us with zero points, 278 -> 271 without).
       if (p->cfg == 8 && 2 * rest <= 256) p->cfg = 12;
+      // Where the rows behind the whole rounds make up (nearly) one round of 128 x 192 tiles - and so would
+      // be three quarters of a round of the wide tile, or more than a round of 128 x 128 tiles - they run
+      // as those (57344 x 8192 at M = 512: 387 against 398 us).
+      if (p->cfg == 0 && nb > 0 && m_tiles <= 512) {
+        const int slots = 512 / m_tiles;
+        const int rest_rb = row_blocks - nb * 16;
+        const int n192 = (rest_rb + 11) / 12;
+        if (rest_rb > 8 * slots && n192 <= slots && 10 * n192 >= 9 * slots) p->cfg = 15;
+      }
       // 6-bit codes for four row blocks do not fit beside the accumulators of the 128 x 256 tile even
       // with a single set refilled octet by octet (as 8-bit codes are): it spills and runs at half the
       // rate of the 128 x 128 ring tile (8192 x 8192, M = 2048, 6 bits: 596 against 281 us).
@@ -384,7 +393,7 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       R = 1 << ((variant - 80) % 3);
       p->mb = 1 << ((variant - 80) / 3);
     } else if (variant >= 64) {
-      if (variant - 64 > 14) return MATGPTQ_EVARIANT;
+      if (variant - 64 > 15) return MATGPTQ_EVARIANT;
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 64;

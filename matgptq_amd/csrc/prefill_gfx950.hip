@@ -741,15 +741,17 @@ prefill_split_kernel(const GemmArgs a, int m_tiles) {
 // `n_big` workgroups take the 128 x 256 tiles of the weight rows below row block `rb_tail`, and
 // the rest of the rows go to workgroups with tiles of half the width, which come last, spread
 // over twice as many CUs and finish in about half the time.
-template <int BITS, int GROUP, bool ZP>
+// (RBW_TAIL 3: the remaining rows as 128 x 192 tiles, where those make up one round of their own and
+// 128 x 128 tiles would not fit one)
+template <int BITS, int GROUP, bool ZP, int RBW_TAIL = 2>
 __global__ void __launch_bounds__(256, 2)
 prefill_tail_kernel(const GemmArgs a, int m_tiles, int n_big, int rb_tail) {
-  static_assert(prefill_lds_halves(4, 8) == prefill_lds_halves(2, 8), "both tiles share one LDS block");
+  static_assert(prefill_lds_halves(4, 8) == prefill_lds_halves(RBW_TAIL, 8), "both tiles share one LDS block");
   __shared__ __align__(16) _Float16 lds[prefill_lds_halves(4, 8)];
   if ((int)blockIdx.x < n_big)
     prefill_body<BITS, GROUP, ZP, 4, 8>(a, blockIdx.x, m_tiles, 0, lds);
   else
-    prefill_body<BITS, GROUP, ZP, 2, 8>(a, blockIdx.x - n_big, m_tiles, rb_tail, lds);
+    prefill_body<BITS, GROUP, ZP, RBW_TAIL, 8>(a, blockIdx.x - n_big, m_tiles, rb_tail, lds);
 }
 
 // The same split of the weight rows in workgroups of eight waves: the 128 x 256 tiles two to a
@@ -807,14 +809,14 @@ hipError_t launch_tail8(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <int GROUP, bool ZP>
+template <int GROUP, bool ZP, int RBW_TAIL = 2>
 hipError_t launch_tail(const GemmArgs& a, hipStream_t stream) {
   const int m_tiles = (a.M + 127) / 128;
   const int nb = prefill_tail_big_tiles(a.row_blocks, m_tiles);
   const int rb_tail = nb * 16;
-  const int n_small = (a.row_blocks - rb_tail + 7) / 8;
+  const int n_small = (a.row_blocks - rb_tail + 4 * RBW_TAIL - 1) / (4 * RBW_TAIL);
   const dim3 grid((nb + n_small) * m_tiles), block(256);
-  hipLaunchKernelGGL((prefill_tail_kernel<kBits, GROUP, ZP>), grid, block, 0, stream, a, m_tiles,
+  hipLaunchKernelGGL((prefill_tail_kernel<kBits, GROUP, ZP, RBW_TAIL>), grid, block, 0, stream, a, m_tiles,
                      nb * m_tiles, rb_tail);
   return hipGetLastError();
 }
@@ -859,6 +861,7 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 12: return launch_tail8<GROUP, ZP>(a, s);      // 128 x 256 in pairs, then a tail of 128 x 128 with K split
     case 13: return launch_split<GROUP, ZP, 3, 8>(a, s);  // 128 x 192, K split in the workgroup
     case 14: return launch_mix<GROUP, ZP>(a, s);          // 128 x 192 and 128 x 128, one round of all slots
+    case 15: return launch_tail<GROUP, ZP, 3>(a, s);      // 128 x 256, then a tail of 128 x 192
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 #endif

@@ -105,7 +105,7 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(15))
+@pytest.mark.parametrize("cfg", range(16))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
@@ -343,6 +343,24 @@ def test_prefill_two_tile_widths_in_one_launch(b, g, zp):
     narrow = lay.run(x, flags=1 | ((64 + 3) << 8))
     assert np.array_equal(y[:, :576], wide[:, :576])
     assert np.array_equal(y[:, 576:], narrow[:, 576:])
+
+
+@pytest.mark.parametrize("b,g,zp", ((4, 128, True), (4, 128, False), (2, 128, True), (8, 128, True), (6, 128, True),
+                                    (4, -1, True)))
+def test_prefill_wide_tiles_with_a_tail_of_192_row_tiles(b, g, zp):
+    # 73 activation tiles: 7 weight tiles of 256 rows make up the whole round (511 workgroups), the other
+    # 29 row blocks go to three tiles of 192 rows (the last one ragged); ragged M.  Each part equals
+    # the launch that uses its width alone.
+    n, k, m = 7 * 256 + 29 * 16, 384, 73 * 128 - 5
+    lay = G.Layer(n, k, b, g, seed=15 + b, zero_points=zp)
+    x = o.make_activations(m, k, seed=15)
+    y = lay.run(x, flags=1 | ((64 + 15) << 8))
+    G.assert_close_to_oracle(y, x, lay.w, f"192-row tail b={b} g={g} zp={zp}")
+    G.assert_regression_bound(y, x, lay.w, f"192-row tail b={b} g={g} zp={zp}")
+    wide = lay.run(x, flags=1 | ((64 + 0) << 8))
+    tail = lay.run(x, flags=1 | ((64 + 9) << 8))
+    assert np.array_equal(y[:, :1792], wide[:, :1792])
+    assert np.array_equal(y[:, 1792:], tail[:, 1792:])
 
 
 def test_prefill_two_tile_widths_forced_where_they_do_not_apply():

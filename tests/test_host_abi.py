@@ -219,7 +219,23 @@ def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True).endswith("cfg12")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 57344, 8192, 2048, True).endswith("cfg0")
-    assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 13312, 8192, 2048, True).endswith("cfg0")   # a round and five eighths
+
+
+def test_planner_gives_three_quarters_of_a_round_to_192_row_tiles():
+    # behind the whole rounds, rows that would be three quarters of a round of the wide tile (and more
+    # than a round of 128 x 128 tiles) are one round of 128 x 192 tiles
+    assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True).endswith("cfg15")
+    assert _lib.describe_plan(4, 128, 57344, 8192, 512, True).endswith("cfg15")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 1024, True).endswith("cfg15")
+    for bits in (2, 3, 8):
+        assert _lib.describe_plan(bits, 128, 14336, 8192, 2048, True).endswith("cfg15")
+    assert _lib.describe_plan(4, 128, 14336, 8192, 2048, True, 3).endswith("cfg15")   # bf16 storage at 4 bits
+    assert not _lib.describe_plan(6, 128, 14336, 8192, 2048, True).endswith("cfg15")  # formats with a tile rule of their own
+    assert not _lib.describe_plan(4, 32, 14336, 8192, 2048, True).endswith("cfg15")
+    # far from a whole round of them, or nothing behind the whole rounds: the plain tile
+    assert _lib.describe_plan(4, 128, 57344, 8192, 768, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 57344, 8192, 2048, True).endswith("cfg0")
 
 
 def test_planner_keeps_small_batches_on_very_wide_layers_off_the_padded_tiles():
