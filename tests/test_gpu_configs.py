@@ -64,10 +64,14 @@ def test_config4_prefill_full_size(name, plan):
 
 
 @pytest.mark.parametrize("name,m,plan", [("o", 512, "prefill b4 g128 zp1 cfg10"), ("o", 1024, "prefill b4 g128 zp1 cfg11"),
-                                         ("down", 500, "prefill b4 g128 zp1 cfg10"), ("down", 1000, "prefill b4 g128 zp1 cfg11")])
+                                         ("down", 500, "prefill b4 g128 zp1 cfg10"), ("down", 1000, "prefill b4 g128 zp1 cfg11"),
+                                         ("qkv", 512, "prefill b4 g128 zp1 cfg13"), ("qkv", 1000, "prefill b4 g128 zp1 cfg14"),
+                                         ("gate_up", 512, "prefill b4 g128 zp1 cfg15")])
 def test_medium_batch_split_tiles_full_size(name, m, plan):
-    # batches of a few hundred rows on the Llama-3-70B layers with 8192 rows: the ring tiles with K
-    # split inside a workgroup of eight waves (down: 112 K tiles per group of waves; ragged M)
+    # batches of a few hundred rows on the Llama-3-70B layers: the ring tiles with K split inside a
+    # workgroup of eight waves (128 x 128, 128 x 256, and 128 x 192 on qkv; down: 112 K tiles per group of
+    # waves; ragged M), both tile widths in one launch (qkv at about a thousand rows) and the wide tile
+    # with a last round of 128 x 192 tiles (gate_up)
     n, k = LLAMA70B[name]
     assert _lib.describe_plan(4, 128, n, k, m, True) == plan
     q, s, z = o.make_layer(n, k, 128, seed=17)
