@@ -74,6 +74,10 @@ int matgptq_glue_attention_split(const void *qkv, const void *cos_table, const v
                                  void *workspace, int64_t M, int heads, int kv_heads,
                                  int head_dim, int64_t max_ctx, int fuse_rotary, void *stream);
 
+/* out[m] (int64) = index of the largest of x[m, 0:n] (fp32, rows contiguous): the first among equals, a NaN
+ * counts as the largest (torch.argmax).  One launch, no workspace.  M <= 65535, n < 2^31. */
+int matgptq_glue_argmax(const void *x, void *out, int64_t M, int64_t n, void *stream);
+
 /* out[M,F] = silu(gate_up[M, 0:F]) * gate_up[M, F:2F].  F % 8 == 0. */
 int matgptq_glue_silu_mul(const void *gate_up, void *out, int64_t M, int64_t F, void *stream);
 

@@ -18,7 +18,7 @@ MAX_CONTEXT = 8192
 
 EXPORTS = ("matgptq_glue_strerror", "matgptq_glue_add_rmsnorm", "matgptq_glue_rope_cache",
            "matgptq_glue_attention", "matgptq_glue_rope_attention", "matgptq_glue_attention_workspace_floats",
-           "matgptq_glue_attention_split", "matgptq_glue_silu_mul")
+           "matgptq_glue_attention_split", "matgptq_glue_silu_mul", "matgptq_glue_argmax")
 
 _lib = None
 
@@ -43,6 +43,7 @@ def load() -> ctypes.CDLL:
     L.matgptq_glue_attention.argtypes = [vp, vp, vp, vp, vp, i64, ci, ci, ci, i64, vp]
     L.matgptq_glue_rope_attention.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, i64, vp]
     L.matgptq_glue_silu_mul.argtypes = [vp, vp, i64, i64, vp]
+    L.matgptq_glue_argmax.argtypes = [vp, vp, i64, i64, vp]
     L.matgptq_glue_attention_split.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, ci, ci, ci, i64, ci, vp]
     L.matgptq_glue_attention_workspace_floats.argtypes = [i64, ci, i64]
     for name in EXPORTS[1:]:
@@ -158,3 +159,11 @@ def silu_mul(gate_up, out) -> None:
     if gate_up.shape != (m, 2 * f):
         raise GlueError("silu_mul: shapes differ")
     _check(load().matgptq_glue_silu_mul(gate_up.data_ptr(), out.data_ptr(), m, f, _stream()))
+
+
+def argmax(x, out) -> None:
+    """out[m] = torch.argmax(x[m]) for fp32 rows x [M, n]; `out` int64 [M]."""
+    if (x.dtype != torch.float32 or out.dtype != torch.int64 or not x.is_cuda or not out.is_cuda
+            or not x.is_contiguous() or not out.is_contiguous() or x.dim() != 2 or out.shape != (x.shape[0],)):
+        raise GlueError("argmax: fp32 [M, n] in, int64 [M] out, contiguous, on the GPU")
+    _check(load().matgptq_glue_argmax(x.data_ptr(), out.data_ptr(), x.shape[0], x.shape[1], _stream()))

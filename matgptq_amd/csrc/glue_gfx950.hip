@@ -503,6 +503,64 @@ silu_mul_kernel(const _Float16* __restrict__ gu, _Float16* __restrict__ out, int
   *reinterpret_cast<half8*>(out + m * F + j * 8) = o;
 }
 
+// Index of the largest value of each row of x [M, n] (fp32): the first one among equals, a NaN counts
+// as the largest, like torch.argmax.  One workgroup per row: the library's reduction spends 38 us in
+// one workgroup of 512 threads on a vocabulary of 128256; sixteen waves with eight 16-byte loads in
+// flight per thread read the same 0.5 MB in a few microseconds.
+constexpr int kArgmaxThreads = 1024;
+__device__ __forceinline__ bool argmax_better(float v, int i, float bv, int bi) {
+  const bool vn = v != v, bn = bv != bv;
+  if (vn != bn) return vn;
+  if (vn) return i < bi;
+  return v > bv || (v == bv && i < bi);
+}
+__global__ void __launch_bounds__(kArgmaxThreads)
+argmax_kernel(const float* __restrict__ x, int64_t* __restrict__ out, int64_t n) {
+  __shared__ float sv[kArgmaxThreads / 64];
+  __shared__ int si[kArgmaxThreads / 64];
+  const float* row = x + (size_t)blockIdx.x * (size_t)n;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  // whole float4 chunks when the row starts on 16 bytes, element by element otherwise and at the end
+  const bool aligned = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  const int chunks = aligned ? (int)(n / 4) : 0;
+  constexpr int kDepth = 8;
+  for (int c0 = threadIdx.x; c0 < chunks; c0 += kArgmaxThreads * kDepth) {
+    float4 v[kDepth];
+#pragma unroll
+    for (int u = 0; u < kDepth; u++) {  // (unconditional: a chunk past the end re-reads the last one, which changes nothing)
+      const int c = c0 + u * kArgmaxThreads;
+      v[u] = reinterpret_cast<const float4*>(row)[c < chunks ? c : chunks - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < kDepth; u++) {
+      const int c = c0 + u * kArgmaxThreads < chunks ? c0 + u * kArgmaxThreads : chunks - 1;
+      const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+      // a thread meets its indices in rising order: "greater" alone keeps the first of equals
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        if (e[k] > best || (e[k] != e[k] && best == best)) { best = e[k]; bi = 4 * c + k; }
+    }
+  }
+  for (int i = chunks * 4 + threadIdx.x; i < n; i += kArgmaxThreads) {
+    const float e = row[i];
+    if (e > best || (e != e && best == best)) { best = e; bi = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (argmax_better(ov, oi, best, bi)) { best = ov; bi = oi; }
+  }
+  if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kArgmaxThreads / 64; w++)
+      if (argmax_better(sv[w], si[w], best, bi)) { best = sv[w]; bi = si[w]; }
+    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;  // (a row of -inf only: nothing was greater than the start value)
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -580,6 +638,15 @@ int matgptq_glue_attention_split(const void* qkv, const void* cos_table, const v
                                                     workspace, M, heads, kv_heads, max_ctx, stream)
                      : launch_attention_split<false>(qkv, k_cache, v_cache, pos, out, cos_table, sin_table,
                                                      workspace, M, heads, kv_heads, max_ctx, stream);
+}
+
+int matgptq_glue_argmax(const void* x, void* out, int64_t M, int64_t n, void* stream) {
+  if (!x || !out) return MATGPTQ_GLUE_ENULL;
+  if (M <= 0 || n <= 0) return MATGPTQ_GLUE_ESHAPE;
+  if (M > 65535 || n > 0x7fffffff) return MATGPTQ_GLUE_ESIZE;
+  hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)M), dim3(kArgmaxThreads), 0, (hipStream_t)stream,
+                     (const float*)x, (int64_t*)out, n);
+  return launch_status();
 }
 
 int matgptq_glue_silu_mul(const void* gate_up, void* out, int64_t M, int64_t F, void* stream) {

@@ -38,6 +38,9 @@ def test_argument_checks_come_before_any_launch():
     assert L.matgptq_glue_attention_split(one, one, one, one, one, one, one, one, 2, 4, 2, 128, 64, 1, None) == -3
     assert L.matgptq_glue_attention_split(one, None, None, one, one, one, one, one, 1, 6, 2, 128, 64, 0, None) == -3
     assert L.matgptq_glue_attention_workspace_floats(2, 4, 65) == 2 * 4 * 2 * 130
+    assert L.matgptq_glue_argmax(None, one, 1, 8, None) == -4
+    assert L.matgptq_glue_argmax(one, one, 0, 8, None) == -3
+    assert L.matgptq_glue_argmax(one, one, 1, 2 ** 31, None) == -8
     assert L.matgptq_glue_silu_mul(one, None, 1, 64, None) == -4
     assert L.matgptq_glue_silu_mul(one, one, 1, 60, None) == -3
     assert b"NULL" in L.matgptq_glue_strerror(-4)

@@ -191,6 +191,32 @@ def test_silu_mul(m, f):
     assert float((out.float() - ref.float()).abs().max()) <= 2e-3 * float(ref.float().abs().max())
 
 
+@pytest.mark.parametrize("m,n", [(1, 128256), (1, 512), (3, 1001), (2, 7), (5, 4096 * 8 + 3)])
+def test_argmax_equals_torch(m, n):
+    # rows of odd length start off 16 bytes from the second row on: those are read element by element
+    from matgptq_amd import _glue
+
+    x = torch.randn(m, n, device=DEV, generator=_gen(n))
+    out = torch.full((m,), -1, device=DEV, dtype=torch.int64)
+    _glue.argmax(x, out)
+    assert torch.equal(out, x.argmax(dim=-1))
+
+
+def test_argmax_takes_the_first_of_equal_values_and_a_nan_before_any_number():
+    from matgptq_amd import _glue
+
+    n = 128256
+    x = torch.zeros(3, n, device=DEV)
+    x[0, 70000] = x[0, 5] = x[0, 128255] = 4.0        # ties: the first index
+    x[1, 99999] = float("nan")                        # a NaN wins over +inf
+    x[1, 7] = float("inf")
+    x[2] = -float("inf")                              # nothing larger than the start value: index 0
+    out = torch.empty(3, device=DEV, dtype=torch.int64)
+    _glue.argmax(x, out)
+    assert out.tolist() == [5, 99999, 0]
+    assert torch.equal(out, x.argmax(dim=-1))
+
+
 def test_wrong_tensors_are_refused():
     from matgptq_amd import _glue
 
@@ -201,6 +227,10 @@ def test_wrong_tensors_are_refused():
         _glue.add_rmsnorm(h, None, h[0, :128], h, 1e-5)
     with pytest.raises(_glue.GlueError):
         _glue.silu_mul(h, torch.zeros(1, 100, device=DEV, dtype=torch.float16))
+    with pytest.raises(_glue.GlueError):
+        _glue.argmax(h, torch.zeros(1, device=DEV, dtype=torch.int64))          # fp16 logits
+    with pytest.raises(_glue.GlueError):
+        _glue.argmax(h.float(), torch.zeros(2, device=DEV, dtype=torch.int64))  # one index per row
 
 
 def _decoder(context=80, seed=5):
