@@ -94,7 +94,7 @@ def main() -> int:
                          "small: launch only the gemv kernel's instantiations for two and for eight batch rows, "
                          "4096->28672 at M=2 and 14336->4096 at M=8.  "
                          "medium: launch only the ring tiles that split K inside the workgroup, 8192->8192 at "
-                         "M=512 and M=1024")
+                         "M=256 (64 x 128 tiles), M=512 and M=1024")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -181,7 +181,7 @@ def main() -> int:
         packed = make_ring(n, k, bits, 1)[0]
         sc, zr = make_aux(n, k)
         plans = []
-        for m in (512, 1024):
+        for m in (256, 512, 1024):
             x = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
             y = torch.empty(m, n, dtype=torch.float16, device=dev)
             with torch.cuda.stream(stream):
@@ -529,25 +529,27 @@ def main() -> int:
             torch.cuda.empty_cache()
         extra["speedup_over_dense_fp16"] = speed
         # ------------------------------------------------ batches of a few hundred rows
-        # (chunked prefill): the Llama-3-70B layers at 4 bits, zero-point form, beside the dense
+        # (chunked prefill): the Llama-3-70B and 8B layers at 4 bits, zero-point form, beside the dense
         # fp16 product on the same GPU; graphs of five launches, median of five replays
-        medium = {}
-        for name, (n, k) in LLAMA3_70B.items():
-            packed = make_ring(n, k, 4, 1)[0]
-            sc, zr = make_aux(n, k)
-            wd = (torch.randn(n, k, device=dev, generator=g) * 0.02).to(torch.float16)
-            for m in (128, 256, 512, 1024):
-                xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
-                ym = torch.empty(m, n, dtype=torch.float16, device=dev)
-                t = timed_graph(lambda: [launch(4, n, k, xm, packed, sc, zr, ym) for _ in range(5)]) / 5
-                t_dense = timed_graph(lambda: [torch.nn.functional.linear(xm, wd) for _ in range(5)]) / 5
-                medium[f"{name}_M{m}"] = {"us": round(t * 1e6, 1), "dense_us": round(t_dense * 1e6, 1),
-                                          "speedup": round(t_dense / t, 2),
-                                          "TFLOPs": round(2.0 * m * n * k / t / 1e12, 1),
-                                          "kernel": _lib.describe_plan(4, GROUP, n, k, m, True)}
-            del packed, wd
-            torch.cuda.empty_cache()
-        extra["medium_batch_llama3_70b_b4"] = medium
+        for table, layers, batches in (("medium_batch_llama3_70b_b4", LLAMA3_70B, (128, 256, 512, 1024)),
+                                       ("medium_batch_llama3_8b_b4", LLAMA3_8B, (256, 512, 768))):
+            medium = {}
+            for name, (n, k) in layers.items():
+                packed = make_ring(n, k, 4, 1)[0]
+                sc, zr = make_aux(n, k)
+                wd = (torch.randn(n, k, device=dev, generator=g) * 0.02).to(torch.float16)
+                for m in batches:
+                    xm = torch.randn(m, k, device=dev, generator=g).to(torch.float16)
+                    ym = torch.empty(m, n, dtype=torch.float16, device=dev)
+                    t = timed_graph(lambda: [launch(4, n, k, xm, packed, sc, zr, ym) for _ in range(5)]) / 5
+                    t_dense = timed_graph(lambda: [torch.nn.functional.linear(xm, wd) for _ in range(5)]) / 5
+                    medium[f"{name}_M{m}"] = {"us": round(t * 1e6, 1), "dense_us": round(t_dense * 1e6, 1),
+                                              "speedup": round(t_dense / t, 2),
+                                              "TFLOPs": round(2.0 * m * n * k / t / 1e12, 1),
+                                              "kernel": _lib.describe_plan(4, GROUP, n, k, m, True)}
+                del packed, wd
+                torch.cuda.empty_cache()
+            extra[table] = medium
         # ---------------------------------------------------------- load time
         # What process_weights_after_loading costs per layer (gate_up of Llama-3-8B, 117 M master
         # codes already in HBM): slice + pack in one kernel (reads 1 byte per code, writes b/8),
@@ -647,6 +649,8 @@ def final_line(headline: dict, roofline: dict, cpu_baseline, extra: dict, extra_
     summary["prefill_b6_b8_min_pct_mfma_peak"] = min(wide) if wide else None
     medium = [v["speedup"] for v in (extra.get("medium_batch_llama3_70b_b4") or {}).values() if "speedup" in v]
     summary["medium_batch_min_speedup_over_dense_fp16"] = min(medium) if medium else None
+    medium = [v["speedup"] for v in (extra.get("medium_batch_llama3_8b_b4") or {}).values() if "speedup" in v]
+    summary["medium_batch_8b_min_speedup_over_dense_fp16"] = min(medium) if medium else None
     summary["decoder_tokens_per_s_graph"] = (extra.get("mixnmatch_decoder_end_to_end") or {}).get("tokens_per_s_graph")
     summary["transformers_tokens_per_s_compiled"] = (extra.get("transformers_end_to_end") or {}).get("tokens_per_s_compiled")
     summary = {k: v for k, v in summary.items() if v is not None}

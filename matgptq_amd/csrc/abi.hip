@@ -90,7 +90,7 @@ size_t decode_lds_bytes(int R, int S, int W, int kc, int64_t M) {
 
 // Automatic choice; the flags word can override it for benchmarks:
 //   bits 8..15 : 0 = automatic, 1 + rsel + 3*shape = decode (rsel: R = 1,2,4; shape: kShapes),
-//                64 + cfg = prefill tile configuration,
+//                64 + cfg = prefill tile configuration 0..15, 89 and 90 = configurations 16 and 17,
 //                80 + rsel + 3*msel = mid-batch kernel (rsel: R = 1,2,4; msel: 16, 32, 64 batch rows)
 //   bits 16..17: decode flavour, 0 = automatic, 1 = burst, 2 = stream
 int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp, uint32_t flags,
@@ -144,9 +144,9 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     // M = 32: 117 us, against 65 on the small tile).
     const bool small_batch_many_rows =
         M <= 64 && t_32 < (11.5 + 3.2 * (double)k_tiles) * (wgs_big > 512 ? (double)wgs_big / 512.0 : 1.0);
-    if (wgs_big >= 288 && small_batch_many_rows) {
+    if (wgs_big > 256 && small_batch_many_rows) {
       p->cfg = 4;
-    } else if (wgs_big >= 288) {
+    } else if (wgs_big > 256) {
       p->cfg = 0;
       // Whole rounds of 512 resident workgroups plus at most half a round: the rows of that
       // fraction go to 128 x 128 tiles, which run last, one per CU, in about a third of a
@@ -170,6 +170,20 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         const int rest_rb = row_blocks - nb * 16;
         const int n192 = (rest_rb + 11) / 12;
         if (rest_rb > 8 * slots && n192 <= slots && 10 * n192 >= 9 * slots) p->cfg = 15;
+      }
+      // Behind ONE whole round, the cheapest of the three tails, in units of a round of the wide tile:
+      // a tile takes its share of the width, times 1.3 (128 rows) or 1.07 (192 rows) for the narrower
+      // tile's lower rate; workgroups that number no more than the CUs sit alone there and finish in 0.7
+      // of that, and 128-row tiles that few run K split in 0.35 (28672 x 4096, behind 105 us for the
+      // whole round: M = 768, 162 / 324 / 216 workgroups, 180 / 176 / 162 us; M = 896, 273 / 546 / 364,
+      // 212 / 215 / 193 us; M = 640, 50 / 100 / 70, 170 / 140 (K split) / 157 us).
+      if (nb > 0 && (int64_t)nb * m_tiles <= 512 && row_blocks > nb * 16 && p->cfg != 12) {
+        const int rest_rb = row_blocks - nb * 16;
+        auto occupancy = [](int64_t n) { return n <= 256 ? 0.7 : (double)((n + 511) / 512); };
+        const int64_t n256 = (int64_t)((rest_rb + 15) / 16) * m_tiles, n128 = (int64_t)((rest_rb + 7) / 8) * m_tiles;
+        const int64_t n192 = (int64_t)((rest_rb + 11) / 12) * m_tiles;
+        const double t256 = occupancy(n256), t128 = occupancy(n128) * 0.5 * 1.3, t192 = occupancy(n192) * 0.75 * 1.07;
+        p->cfg = t192 < t256 && t192 < t128 ? 15 : t128 < t256 ? 8 : 0;
       }
       // 6-bit codes for four row blocks do not fit beside the accumulators of the 128 x 256 tile even
       // with a single set refilled octet by octet (as 8-bit codes are): it spills and runs at half the
@@ -224,8 +238,19 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
         // ... and where those leave slots empty while 128 x 128 tiles would need a second round, both
         // widths in one launch take every slot once (10240 x 8192 at M = 1024: 432 tiles of 192 rows on
         // 512 slots; 256 of them and 256 of 128 rows instead)
+        // (the wide tiles of the mix must not number more than the CUs, or some CUs get two of them and
+        // finish no earlier than with 128 x 192 tiles alone: 28672 x 4096 at M = 384, 324 wide tiles: 93
+        // against 89 us)
         int narrow = 0;
-        if (prefill_mix_wide_tiles(row_blocks, m_tiles, &narrow) > 0) p->cfg = 14;
+        const int wide = prefill_mix_wide_tiles(row_blocks, m_tiles, &narrow);
+        if (wide > 0 && wide * m_tiles <= 256) p->cfg = 14;
+      } else if (wgs_big <= 512 && fits_192 && p->cfg == 0) {
+        // One round of the 128 x 256 tile that leaves slots empty, while 128 x 192 tiles would need a
+        // second round: both widths in one launch, a wide and a narrow tile on every CU (28672 x 4096 at
+        // M = 512: 448 wide tiles on 512 slots 122 us, 256 wide and 256 narrow 104).
+        int narrow = 0;
+        const int wide = prefill_mix_widest_tiles(row_blocks, m_tiles, &narrow);
+        if (wide > 0 && wide * m_tiles <= 256) p->cfg = 17;
       }
     } else {
       // Below that, the cheapest of four by a cost model fitted to measurements on MI355X
@@ -252,16 +277,23 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       double best = t_128 < t_32 ? t_128 : t_32;
       // Ring tiles that sit one per CU run K in two halves inside a workgroup of eight waves (two
       // per SIMD, as two workgroups would bring): 128 x 128 while those tiles number at most the
-      // CUs, 3 us + 1.0 .. 1.12 per K tile (M = 512: 8192 x 8192 73 against 87 us on the staged
-      // 64 x 256 tile, 8192 x 28672 249 against 298; 4096 x 4096 at M = 1024 40 against 48); 128 x 256 where
+      // CUs, 3 us + 0.74 .. 0.98 per K tile, more as more of the CUs are taken (M = 512: 8192 x 8192 66
+      // against 87 us on the staged 64 x 256 tile, 8192 x 28672 249 against 298; 4096 x 4096 at M = 1024 40 against 48); 128 x 256 where
       // only these number at most the CUs, 5 us + 1.4 .. 1.65 per K tile (8192 x 8192 at M = 1024 111
       // against 125 us on 128 x 128 tiles two per CU, 8192 x 28672 366 against 440), for the formats
       // whose registers fit that tile (bf16 storage: all but 3 and 6 bits and group size 32 -
       // 8192 x 8192 at M = 1024 116 against 128 us at 4 bits, 127 against 148 at 8).
       const bool bf16 = (flags & MATGPTQ_FLAG_BF16) != 0;
       if (wgs_128 <= 256) {
-        const double t = 3.0 + kt * (1.0 + 0.12 * (double)wgs_128 / 256.0);
+        const double wide_codes = bits == 8 ? 1.1 : 1.0;  // (8-bit codes: 24 against 22 us per 32 K tiles)
+        const double t = 3.0 + kt * wide_codes * (0.66 + 0.32 * (double)wgs_128 / 256.0);
         if (t < best) { best = t; p->cfg = 10; }
+        // ... and 64 x 128 tiles the same way where twice as many workgroups still number at most the
+        // CUs, 4.5 us + 0.5 .. 0.64 per K tile (4096 x 4096 at M = 512: 25 against 30 us, 4096 x 14336:
+        // 74 against 88; 6144 x 4096 at M = 256: 25 against 31)
+        const int64_t wgs_64s = ((N + 127) / 128) * ((M + 63) / 64);
+        const double t6 = 4.5 + kt * (bits == 8 ? 1.2 : 1.0) * (bf16 ? 1.05 : 1.0) * (0.45 + 0.19 * (double)wgs_64s / 256.0);
+        if (wgs_64s <= 256 && t6 < best) { best = t6; p->cfg = 16; }
       } else if (wgs_big <= 256 && bits != 6 && !(bf16 && (bits == 3 || group_size == 32)) && !(group_size == 32 && zp)) {
         const double t = 5.0 + kt * (wgs_big > 192 ? 1.65 : 1.4);
         if (t < best) { best = t; p->cfg = 11; }
@@ -386,8 +418,12 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   }
   if (variant != 0) {
     if (variant >= 100) return MATGPTQ_EVARIANT;
-    if (variant >= 80) {
-      if (variant - 80 > 8) return MATGPTQ_EVARIANT;
+    if (variant >= 89) {  // prefill tiles 16 and up
+      if (variant - 89 > 1) return MATGPTQ_EVARIANT;
+      p->decode = false;
+      p->skinny = false;
+      p->cfg = variant - 89 + 16;
+    } else if (variant >= 80) {
       p->decode = false;
       p->skinny = true;
       R = 1 << ((variant - 80) % 3);

@@ -61,7 +61,11 @@ constexpr int kXsPitch = kXs + MATGPTQ_XPAD;  // halves per LDS row
 // Two waves per SIMD (256 registers each) whenever the accumulators leave room for the rest:
 // one wave alone cannot keep the matrix pipe busy.  The tile whose accumulators take half of
 // that budget runs the ring loop below (activations straight into LDS, one operand set).
-constexpr bool prefill_lean(int rbw, int mt) { return (rbw == 4 || rbw == 3 || rbw == 2) && mt == 8; }
+// (64 batch rows x 128 weight rows run the same loop: the K-split tile of batches whose 128-row tiles
+// would leave half of the CUs idle)
+constexpr bool prefill_lean(int rbw, int mt) {
+  return ((rbw == 4 || rbw == 3 || rbw == 2) && mt == 8) || (rbw == 2 && mt == 4);
+}
 constexpr int prefill_min_waves(int rbw, int mt) { return rbw * mt * 4 < 128 || prefill_lean(rbw, mt) ? 2 : 1; }
 
 // LDS of a workgroup, in halves: the ring loop keeps four unpadded buffers of 64 columns, the
@@ -287,12 +291,15 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
     _Float16* const ring1 = lds + TM * kXs;
     _Float16* const ring2 = lds + 2 * TM * kXs;
     _Float16* const ring3 = lds + 3 * TM * kXs;
-    static_assert(TM == 128, "the copy below moves 32 rows per wave");
-    // this lane's part of a copy: rows wave*32 + i*8 + lane/8, LDS chunk lane%8
-    uint32_t dma_voff[4];
+    static_assert(TM % 32 == 0, "a wave copies a quarter of the rows, eight per instruction");
+    constexpr int kRowsPerWave = TM / 4;
+    constexpr int kD = kRowsPerWave / 8;  // copy instructions of a wave per half tile
+    // this lane's part of a copy: rows wave*kRowsPerWave + i*8 + lane/8, LDS chunk lane%8
+    static_assert(kD <= 4, "offsets of at most four copies are kept");
+    uint32_t dma_voff[4];  // kD of them in use (a bound that depends on the tile does not pass the host compilation)
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int r = wave * 32 + i * 8 + (lane >> 3);
+    for (int i = 0; i < kD; i++) {
+      const int r = wave * kRowsPerWave + i * 8 + (lane >> 3);
       const int c = (lane & 7) ^ ((r >> 1) & 7);
       const uint32_t m = (uint32_t)(m0 + r);
       dma_voff[i] = m < (uint32_t)a.M ? (m * (uint32_t)a.K + c * 8) * 2u : x_bytes;
@@ -313,18 +320,18 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
         // no difference in pairs or in workgroups of four waves: those keep the intrinsic.)
         const uint64_t xa = (uint64_t)(uintptr_t)a.x;
         const u32x4 xd = {(uint32_t)xa, (uint32_t)(xa >> 32) & 0xffffu, valid ? x_bytes : 0u, 0x00020000u};
-        const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(ring + wave * 32 * kXs);
+        const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(ring + wave * kRowsPerWave * kXs);
 #pragma unroll
-        for (int i = 0; i < 4; i++)  // m0: LDS address of the wave's 8 rows; one wait state before its use
+        for (int i = 0; i < kD; i++)  // m0: LDS address of the wave's 8 rows; one wait state before its use
           asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                        :
                        : "s"(base + i * 8 * kXs * 2), "v"(dma_voff[i]), "s"(xd), "s"((uint32_t)ih * (kXs * 2))
                        : "memory", "m0");
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < kD; i++)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(
-              xres, (__attribute__((address_space(3))) void*)(ring + (wave * 32 + i * 8) * kXs), 16, dma_voff[i],
+              xres, (__attribute__((address_space(3))) void*)(ring + (wave * kRowsPerWave + i * 8) * kXs), 16, dma_voff[i],
               (uint32_t)ih * (kXs * 2), 0, 0);
       }
     };
@@ -448,8 +455,8 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       //   r3 loads fewer: the smaller count is used for every tile (a stricter wait, on loads that are
       //   more than a tile old).  Barrier B of tile t needs D(2t+2), issued behind barrier A of tile t-1;
       //   issued after it: R1 R2 D R3 S | R0 D R1 R2 (more at t = 0).
-      constexpr int kWaitA = 8 + 2 * r0 + r1 + r2 + r3 + 2 * kS;
-      constexpr int kWaitB = 8 + r0 + 2 * r1 + 2 * r2 + r3 + kS;
+      constexpr int kWaitA = 2 * kD + 2 * r0 + r1 + r2 + r3 + 2 * kS;
+      constexpr int kWaitB = 2 * kD + r0 + 2 * r1 + 2 * r2 + r3 + kS;
       dma(ring0, 0);
       dma(ring1, 1);
       dma(ring2, 2);
@@ -460,7 +467,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       refill(J3{}, 0);
       load_aux(scur, zcur, 0);
       load_aux(snxt, znxt, 1);
-      wait_and_meet(std::integral_constant<int, 12 + r0 + r1 + r2 + r3 + 2 * kS>{});  // D0 has landed
+      wait_and_meet(std::integral_constant<int, 3 * kD + r0 + r1 + r2 + r3 + 2 * kS>{});  // D0 has landed
 #pragma unroll
       for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
       auto stile = [&](int kb, uint32_t (&sc)[RBW][GPT], uint32_t (&zc)[RBW][GPT], _Float16* ra, _Float16* rb,
@@ -500,7 +507,7 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
       dma(ring3, 3);
       load_weights(wcur, scur, zcur, 0);
       load_weights(wnxt, snxt, znxt, 1);
-      wait_and_meet(std::integral_constant<int, 12 + 2 * kW>{});  // D0 has landed
+      wait_and_meet(std::integral_constant<int, 3 * kD + 2 * kW>{});  // D0 has landed
   #pragma unroll
       for (int i = 0; i < MT; i++) ring_frag(bv[i], ring0, i, 0);
       // one tile; ra / rb: the rings of its two half tiles, rn: the ring of the next tile's first
@@ -510,12 +517,12 @@ __device__ __forceinline__ void prefill_body(const GemmArgs& a, int lid, int m_t
                        _Float16* ra, _Float16* rb, _Float16* rn) {
         dstep(wc, sc, zc, J0{}, ra, 1);
         // needs D(2kb+1); younger in steady state: W(kb) D(2kb+2) D(2kb+3) W(kb+1)
-        wait_and_meet(std::integral_constant<int, 8 + 2 * kW>{});
+        wait_and_meet(std::integral_constant<int, 2 * kD + 2 * kW>{});
         dma(ra, 2 * kb + 4);  // every wave is past its reads of ra
         dstep(wc, sc, zc, J1{}, rb, 0);
         dstep(wc, sc, zc, J2{}, rb, 1);
         // needs D(2kb+2); younger: D(2kb+3) W(kb+1) D(2kb+4)
-        wait_and_meet(std::integral_constant<int, 8 + kW>{});
+        wait_and_meet(std::integral_constant<int, 2 * kD + kW>{});
         dma(rb, 2 * kb + 5);
         dstep(wc, sc, zc, J3{}, rn, 0);
       };
@@ -821,6 +828,22 @@ hipError_t launch_tail(const GemmArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// 128 x 256 and 128 x 192 tiles in one round of all slots (prefill_mix_widest_tiles): the kernel of the
+// 192-row tail, with the wide tiles counted by the mix instead of by whole rounds
+template <int GROUP, bool ZP>
+hipError_t launch_mix_widest(const GemmArgs& a, hipStream_t stream) {
+  const int m_tiles = (a.M + 127) / 128;
+  int narrow = 0;
+  const int wide = prefill_mix_widest_tiles(a.row_blocks, m_tiles, &narrow);
+  // (forced on a shape the mix does not apply to: 128 x 192 tiles only)
+  const int rb_tail = wide * 16;
+  const int n_small = wide > 0 ? narrow : (a.row_blocks + 11) / 12;
+  const dim3 grid((wide + n_small) * m_tiles), block(256);
+  hipLaunchKernelGGL((prefill_tail_kernel<kBits, GROUP, ZP, 3>), grid, block, 0, stream, a, m_tiles,
+                     wide * m_tiles, rb_tail);
+  return hipGetLastError();
+}
+
 template <int GROUP, bool ZP, int RBW, int MT>
 hipError_t launch_cfg(const GemmArgs& a, hipStream_t stream) {
   const int n_tiles = (a.row_blocks + 4 * RBW - 1) / (4 * RBW);
@@ -862,6 +885,8 @@ hipError_t launch_shape(const GemmArgs& a, int cfg, hipStream_t s) {
     case 13: return launch_split<GROUP, ZP, 3, 8>(a, s);  // 128 x 192, K split in the workgroup
     case 14: return launch_mix<GROUP, ZP>(a, s);          // 128 x 192 and 128 x 128, one round of all slots
     case 15: return launch_tail<GROUP, ZP, 3>(a, s);      // 128 x 256, then a tail of 128 x 192
+    case 16: return launch_split<GROUP, ZP, 2, 4>(a, s);  // 64 x 128, K split in the workgroup
+    case 17: return launch_mix_widest<GROUP, ZP>(a, s);   // 128 x 256 and 128 x 192, one round of all slots
     default: return launch_cfg<GROUP, ZP, 4, 2>(a, s);  // 32 x 256
   }
 #endif

@@ -66,12 +66,13 @@ def test_config4_prefill_full_size(name, plan):
 @pytest.mark.parametrize("name,m,plan", [("o", 512, "prefill b4 g128 zp1 cfg10"), ("o", 1024, "prefill b4 g128 zp1 cfg11"),
                                          ("down", 500, "prefill b4 g128 zp1 cfg10"), ("down", 1000, "prefill b4 g128 zp1 cfg11"),
                                          ("qkv", 512, "prefill b4 g128 zp1 cfg13"), ("qkv", 1000, "prefill b4 g128 zp1 cfg14"),
-                                         ("gate_up", 512, "prefill b4 g128 zp1 cfg15")])
+                                         ("gate_up", 512, "prefill b4 g128 zp1 cfg15"),
+                                         ("o", 250, "prefill b4 g128 zp1 cfg16"), ("down", 250, "prefill b4 g128 zp1 cfg16")])
 def test_medium_batch_split_tiles_full_size(name, m, plan):
     # batches of a few hundred rows on the Llama-3-70B layers: the ring tiles with K split inside a
     # workgroup of eight waves (128 x 128, 128 x 256, and 128 x 192 on qkv; down: 112 K tiles per group of
-    # waves; ragged M), both tile widths in one launch (qkv at about a thousand rows) and the wide tile
-    # with a last round of 128 x 192 tiles (gate_up)
+    # waves; ragged M), both tile widths in one launch (qkv at about a thousand rows), the wide tile
+    # with a last round of 128 x 192 tiles (gate_up), and 64 x 128 tiles with K split (250 rows)
     n, k = LLAMA70B[name]
     assert _lib.describe_plan(4, 128, n, k, m, True) == plan
     q, s, z = o.make_layer(n, k, 128, seed=17)
@@ -81,11 +82,33 @@ def test_medium_batch_split_tiles_full_size(name, m, plan):
     y = G.gemm(4, 128, n, k, G.to_dev(x), packed, sc, zr)
     torch.cuda.synchronize()
     assert bool(torch.isfinite(y.float()).all())
-    tiles = (m + 127) // 128
-    rows = np.array(sorted({min(t * 128 + (37 * t + 5) % 128, m - 1) for t in range(tiles)} | {0, m - 1}))
+    tiles = (m + 63) // 64  # a row of every 64: one or two per activation tile
+    rows = np.array(sorted({min(t * 64 + (37 * t + 5) % 64, m - 1) for t in range(tiles)} | {0, m - 1}))
     yr = y[torch.from_numpy(rows).to(G.DEV)].cpu().numpy()
     ref, bound = G.oracle_product_in_chunks(q, s, z, 4, 128, x[rows])
     G.assert_close_to_reference(yr, ref, bound, f"70B {name} M={m}")
+
+
+@pytest.mark.parametrize("name,m,plan", [("gate_up", 512, "prefill b4 g128 zp1 cfg17"), ("gate_up", 760, "prefill b4 g128 zp1 cfg15"),
+                                         ("o", 500, "prefill b4 g128 zp1 cfg16"), ("down", 512, "prefill b4 g128 zp1 cfg16")])
+def test_medium_batch_llama3_8b_full_size(name, m, plan):
+    # batches of a few hundred rows on the Llama-3-8B layers: 128 x 256 and 128 x 192 tiles in one round
+    # (gate_up at 512 rows), the wide tile with 216 tiles of 192 rows behind its one round (760 rows), and
+    # 64 x 128 tiles with K split in the workgroup (o; down: 56 K tiles per group of waves)
+    n, k = LLAMA8B[name]
+    assert _lib.describe_plan(4, 128, n, k, m, True) == plan
+    q, s, z = o.make_layer(n, k, 128, seed=19)
+    x = o.make_activations(m, k, seed=m)
+    packed = G.pack_device(q, 4, True)
+    sc, zr = G.reorder_device(s, n, k, 128), G.reorder_device(z, n, k, 128)
+    y = G.gemm(4, 128, n, k, G.to_dev(x), packed, sc, zr)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(y.float()).all())
+    tiles = (m + 63) // 64
+    rows = np.array(sorted({min(t * 64 + (37 * t + 5) % 64, m - 1) for t in range(tiles)} | {0, m - 1}))
+    yr = y[torch.from_numpy(rows).to(G.DEV)].cpu().numpy()
+    ref, bound = G.oracle_product_in_chunks(q, s, z, 4, 128, x[rows])
+    G.assert_close_to_reference(yr, ref, bound, f"8B {name} M={m}")
 
 
 @pytest.mark.parametrize("m", (1, 2, 4))

@@ -105,11 +105,17 @@ def test_prefill_parity(b, g, zp):
         G.assert_close_to_oracle(lay.run(x), x, lay.w, f"prefill b={b} g={g} zp={zp} M={m}")
 
 
-@pytest.mark.parametrize("cfg", range(16))
+def _tile(cfg):
+    # flags that force prefill tile configuration `cfg`: 64 + cfg up to 15, 89 for configuration 16
+    return 1 | ((64 + cfg if cfg < 16 else 89 + cfg - 16) << 8)
+
+
+@pytest.mark.parametrize("cfg", range(18))
 def test_prefill_every_tile_configuration(cfg):
     lay = G.Layer(1040, 1024, 4, 128, seed=3)
     x = o.make_activations(300, 1024, seed=1)
-    G.assert_close_to_oracle(lay.run(x, flags=1 | ((64 + cfg) << 8)), x, lay.w, f"cfg {cfg}")
+    G.assert_close_to_oracle(lay.run(x, flags=_tile(cfg)), x, lay.w, f"cfg {cfg}")
+    assert _lib.describe_plan(4, 128, 1040, 1024, 300, True, _tile(cfg)).endswith(f"cfg{cfg}")
 
 
 def _decode_variants():
@@ -138,25 +144,25 @@ def test_prefill_ring_tile_every_format(b, g, zp):
 def test_prefill_split_tiles_every_format(b, g, zp):
     # K in two halves inside a workgroup of eight waves, each group with a ring of its own and
     # the same hand-counted waits; the second group's sums cross LDS at the end.  Seven K tiles
-    # (the second group walks one tile fewer), ragged M and N; both tile widths.
+    # (the second group walks one tile fewer), ragged M and N; every tile shape.
     n, k, m = 304, 128 * 7, 200
     lay = G.Layer(n, k, b, g, seed=29 * b + (g & 7), zero_points=zp)
     x = o.make_activations(m, k, seed=b + 2)
-    for cfg in (10, 11, 13):
-        flags = 1 | ((64 + cfg) << 8)
+    for cfg in (10, 11, 13, 16):
+        flags = _tile(cfg)
         for _ in range(2):
             G.assert_close_to_oracle(lay.run(x, flags=flags), x, lay.w, f"split tile cfg{cfg} b={b} g={g} zp={zp}")
         assert _lib.describe_plan(b, g, n, k, m, zp, flags).endswith(f"cfg{cfg}")
 
 
 @pytest.mark.parametrize("k_tiles", (1, 2, 3, 10))
-@pytest.mark.parametrize("cfg", (10, 11, 13))
+@pytest.mark.parametrize("cfg", (10, 11, 13, 16))
 def test_prefill_split_tiles_short_and_even_walks(cfg, k_tiles):
     # one K tile leaves the second group with nothing but zeros; two give each group a single trip
     n, k, m = 528, 128 * k_tiles, 130
     lay = G.Layer(n, k, 4, 128, seed=k_tiles)
     x = o.make_activations(m, k, seed=cfg)
-    G.assert_close_to_oracle(lay.run(x, flags=1 | ((64 + cfg) << 8)), x, lay.w, f"split cfg{cfg} {k_tiles} K tiles")
+    G.assert_close_to_oracle(lay.run(x, flags=_tile(cfg)), x, lay.w, f"split cfg{cfg} {k_tiles} K tiles")
 
 
 def test_prefill_split_tile_agrees_with_the_plain_tile_closely():
@@ -165,8 +171,8 @@ def test_prefill_split_tile_agrees_with_the_plain_tile_closely():
     lay = G.Layer(n, k, 4, 128, seed=8)
     x = o.make_activations(m, k, seed=9)
     plain = lay.run(x, flags=1 | (67 << 8)).astype(np.float64)
-    for cfg in (10, 11, 13):
-        y = lay.run(x, flags=1 | ((64 + cfg) << 8)).astype(np.float64)
+    for cfg in (10, 11, 13, 16):
+        y = lay.run(x, flags=_tile(cfg)).astype(np.float64)
         assert np.max(np.abs(y - plain)) <= 2.0 ** -9 * np.max(np.abs(plain))
         assert np.mean(y == plain) > 0.9
 
@@ -363,6 +369,25 @@ def test_prefill_wide_tiles_with_a_tail_of_192_row_tiles(b, g, zp):
     assert np.array_equal(y[:, 1792:], tail[:, 1792:])
 
 
+@pytest.mark.parametrize("b,g,zp", ((4, 128, True), (4, 128, False), (2, 128, True), (3, 128, True), (8, 128, True),
+                                    (4, -1, True), (4, 32, False)))
+def test_prefill_widest_tile_mixed_with_192_row_tiles(b, g, zp):
+    # 99 row blocks, 73 activation tiles (7 slots per column): 4 tiles of 256 rows take the first 64 row
+    # blocks, 3 tiles of 192 rows the other 35 (the last one ragged); ragged M.  Each part equals the
+    # launch that uses its width alone.
+    n, k, m = 99 * 16, 384, 73 * 128 - 5
+    lay = G.Layer(n, k, b, g, seed=16 + b, zero_points=zp)
+    x = o.make_activations(m, k, seed=16)
+    assert _lib.describe_plan(b, g, n, k, m, zp, _tile(17)).endswith("cfg17")
+    y = lay.run(x, flags=_tile(17))
+    G.assert_close_to_oracle(y, x, lay.w, f"256 and 192 rows b={b} g={g} zp={zp}")
+    G.assert_regression_bound(y, x, lay.w, f"256 and 192 rows b={b} g={g} zp={zp}")
+    wide = lay.run(x, flags=_tile(0))
+    narrow = lay.run(x, flags=_tile(9))
+    assert np.array_equal(y[:, :1024], wide[:, :1024])
+    assert np.array_equal(y[:, 1024:], narrow[:, 1024:])
+
+
 def test_prefill_two_tile_widths_forced_where_they_do_not_apply():
     # one round of narrow tiles is enough here: the launch degenerates to those
     n, k, m = 304, 128 * 7, 200
@@ -370,6 +395,8 @@ def test_prefill_two_tile_widths_forced_where_they_do_not_apply():
     x = o.make_activations(m, k, seed=3)
     y = lay.run(x, flags=1 | ((64 + 14) << 8))
     assert np.array_equal(y, lay.run(x, flags=1 | ((64 + 3) << 8)))
+    # ... and the mix of 256 and 192 rows to tiles of 192 rows
+    assert np.array_equal(lay.run(x, flags=_tile(17)), lay.run(x, flags=_tile(9)))
 
 
 def test_llama3_70b_qkv_at_1024_rows_takes_both_widths():
@@ -539,7 +566,7 @@ def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
     x = np.eye(k, dtype=np.float32)
     pk = G.pack_device(q, b, True)
     w = o.dequantize_bf16(q, s, z, b, g)
-    for cfg in (64, 67, 73, 72, 66, 74, 75, 76, 77, 80, 84, 88):
+    for cfg in (64, 67, 73, 72, 66, 74, 75, 76, 77, 89, 90, 80, 84, 88):
         y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | (cfg << 8))
         assert np.array_equal(y, w.T), (b, zp, cfg)
 

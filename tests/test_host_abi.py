@@ -214,12 +214,33 @@ def test_describe_plan_regimes():
 
 def test_planner_takes_the_tail_split_for_a_fraction_of_a_round():
     # 640 tiles of 128 x 256 are one round of 512 resident workgroups and a quarter: the rows of
-    # the quarter go to narrower tiles; whole rounds, or more than half a round left over, keep the
-    # plain tile
+    # the quarter go to narrower tiles; whole rounds keep the plain tile
     assert _lib.describe_plan(4, 128, 10240, 8192, 2048, True).endswith("cfg12")
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True).endswith("cfg0")
     assert _lib.describe_plan(4, 128, 57344, 8192, 2048, True).endswith("cfg0")
-    assert _lib.describe_plan(4, 128, 13312, 8192, 2048, True).endswith("cfg0")   # a round and five eighths
+    # behind one whole round the cheapest tail by workgroup counts: a round and five eighths (320 wide
+    # tiles left, or 640 of 128 rows, or 432 of 192 rows) ends on 128 x 192 tiles
+    assert _lib.describe_plan(4, 128, 13312, 8192, 2048, True).endswith("cfg15")
+    # 28672 x 4096 behind its one round: 216 tiles of 192 rows sit alone on their CUs (M = 768), 100 of
+    # 128 rows run K split (M = 640), 364 of 192 rows beat 273 wide and 546 narrow ones (M = 896)
+    assert _lib.describe_plan(4, 128, 28672, 4096, 768, True).endswith("cfg15")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 640, True).endswith("cfg12")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 896, True).endswith("cfg15")
+
+
+def test_planner_mixes_the_widest_tile_with_192_rows_where_one_round_of_it_leaves_slots_empty():
+    # 448 tiles of 128 x 256 on 512 slots, 600 of 128 x 192: 256 of the first and 256 of the second
+    assert _lib.describe_plan(4, 128, 28672, 4096, 512, True).endswith("cfg17")
+    assert _lib.describe_plan(4, 128, 14336, 8192, 1024, True).endswith("cfg17")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 512, True, 1 | (90 << 8)).endswith("cfg17")
+    # formats that do not take the 128 x 256 tile keep their own choice
+    assert not _lib.describe_plan(6, 128, 28672, 4096, 512, True).endswith("cfg17")
+    assert not _lib.describe_plan(4, 32, 28672, 4096, 512, True).endswith("cfg17")
+    # the mixes need their wide tiles to number at most the CUs: 324 of 192 rows here, so 192 rows alone
+    assert _lib.describe_plan(4, 128, 28672, 4096, 384, True).endswith("cfg9")
+    # a few more 128 x 256 tiles than CUs (280) are a large batch too: one round of two widths
+    assert _lib.describe_plan(4, 128, 14336, 8192, 640, True).endswith("cfg14")
+    assert _lib.describe_plan(4, 128, 10240, 8192, 896, True).endswith("cfg14")
 
 
 def test_planner_gives_three_quarters_of_a_round_to_192_row_tiles():
@@ -254,7 +275,7 @@ def test_planner_takes_192_row_tiles_where_they_fill_one_round_better():
         assert _lib.describe_plan(bits, 128, 6144, 4096, 2048, True).endswith("cfg9")
     assert _lib.describe_plan(4, 32, 6144, 4096, 2048, False).endswith("cfg9")
     assert _lib.describe_plan(4, 128, 6144, 4096, 2560, True).endswith("cfg0")
-    assert _lib.describe_plan(4, 128, 7168, 4096, 2048, True).endswith("cfg0")
+    assert _lib.describe_plan(4, 128, 7168, 4096, 2048, True).endswith("cfg17")  # 448 wide tiles: mixed with 192 rows
 
 
 def test_planner_mixes_two_tile_widths_where_neither_fills_the_one_round():
@@ -293,6 +314,29 @@ def test_planner_splits_k_in_the_workgroup_where_ring_tiles_would_sit_one_per_cu
     assert _lib.describe_plan(4, 128, 4096, 2048, 1024, True).endswith("cfg10")
     assert _lib.describe_plan(4, 128, 4096, 1024, 1024, True).endswith("cfg10")
     assert _lib.describe_plan(4, 128, 4096, 1024, 512, True).endswith("cfg4")
+
+
+def test_planner_takes_64_row_split_tiles_where_128_row_ones_leave_half_of_the_cus_idle():
+    # 64 x 128 tiles, K in two halves inside the workgroup, while they number at most the CUs
+    assert _lib.describe_plan(4, 128, 4096, 4096, 512, True).endswith("cfg16")
+    assert _lib.describe_plan(4, 128, 6144, 4096, 256, True).endswith("cfg16")
+    assert _lib.describe_plan(4, 128, 4096, 14336, 512, True).endswith("cfg16")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 64, True).endswith("cfg16")
+    assert _lib.describe_plan(4, 32, 4096, 4096, 512, True).endswith("cfg16")      # every format
+    assert _lib.describe_plan(4, -1, 4096, 4096, 512, False).endswith("cfg16")
+    assert _lib.describe_plan(4, 128, 4096, 4096, 512, True, 3).endswith("cfg16")  # bf16 storage
+    assert _lib.describe_plan(8, 128, 6144, 4096, 192, True).endswith("cfg16")
+    # more of them than CUs: the 128-row tile
+    assert _lib.describe_plan(4, 128, 6144, 4096, 384, True).endswith("cfg10")
+    assert _lib.describe_plan(4, 128, 4096, 14336, 768, True).endswith("cfg10")
+    assert _lib.describe_plan(4, 128, 28672, 4096, 128, True).endswith("cfg10")
+    # smaller batches stay with the mid-batch kernel while its workgroups fit their rounds
+    assert _lib.describe_plan(4, 128, 4096, 4096, 192, True).startswith("midbatch")
+    assert _lib.describe_plan(8, 128, 6144, 4096, 96, True).startswith("midbatch")
+    # the forced variant: 89
+    assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 1 | (89 << 8)).endswith("cfg16")
+    with pytest.raises(_lib.MatGPTQError):
+        _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 1 | (91 << 8))
 
 
 def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
