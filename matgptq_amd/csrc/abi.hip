@@ -569,9 +569,10 @@ const char* matgptq_strerror(int code) {
 
 // The kernels that read master-resident bit planes themselves: the gemv kernel in its two shapes
 // built for them, and the mid-batch kernel.
-// (the gemv kernel reads the planes up to four batch rows)
+// (the gemv kernel reads the planes in every batch size it is planned for: one to four rows, and five
+// to eight with one scale per tile or row)
 static bool plan_reads_planes(const Plan& p, int64_t M) {
-  return (p.gemv && M <= kGemvMaxM && (p.shape == 1 || p.shape == 2)) || p.skinny;
+  return (p.gemv && M <= kGemvEightMaxM && (p.shape == 1 || p.shape == 2)) || p.skinny;
 }
 
 // checks, plan, launch; `master_planes`: the weight operand is master-resident bit planes and

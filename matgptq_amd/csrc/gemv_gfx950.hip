@@ -492,10 +492,10 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
   if (a.M <= 4)
     return zp ? launch_shape<true, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream)
               : launch_shape<false, GROUP, 4, MASTER>(a, shape, W, lds_pad, stream);
-  // five to eight batch rows: pre-sliced tiles with one scale per tile or row
-  if constexpr (GROUP != 32 && !MASTER)
-    return zp ? launch_shape<true, GROUP, 8, false>(a, shape, W, lds_pad, stream)
-              : launch_shape<false, GROUP, 8, false>(a, shape, W, lds_pad, stream);
+  // five to eight batch rows: one scale per tile or row
+  if constexpr (GROUP != 32)
+    return zp ? launch_shape<true, GROUP, 8, MASTER>(a, shape, W, lds_pad, stream)
+              : launch_shape<false, GROUP, 8, MASTER>(a, shape, W, lds_pad, stream);
   return hipErrorInvalidValue;
 }
 
@@ -504,8 +504,8 @@ hipError_t launch_storage(const GemmArgs& a, int shape, int W, size_t lds_pad, h
 // Entry of this translation unit.  shape: index into the (T, R) table above; W: waves per
 // workgroup (1..16); lds_pad: dynamic LDS to ask for when it exceeds what the kernel needs
 // (limits how many workgroups share a CU); master: `a.packed` holds master-resident bit planes
-// (shapes 1 and 2); group sizes 32 and -1: shapes 1 and 2.  M <= 4; five to eight batch rows on
-// pre-sliced tiles with group size 128 or -1, shapes 1 and 2.
+// (shapes 1 and 2); group sizes 32 and -1: shapes 1 and 2.  M <= 4; five to eight batch rows with
+// group size 128 or -1, shapes 1 and 2.
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
 #if MATGPTQ_BF16

@@ -99,18 +99,40 @@ def test_midbatch_kernel_reads_the_planes_itself(b, g, m):
     planes = planes_device(q)
     sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
     x = o.make_activations(m, k, seed=m)
-    # (five to eight batch rows of a pre-sliced layer this small go to the gemv kernel, which reads the
-    # planes up to four: on planes they take the mid-batch kernel, forced here for the comparison)
+    # (five to eight batch rows of a layer this small go to the gemv kernel: the mid-batch kernel is
+    # forced for them)
     flags = 1 | (82 << 8) if 5 <= m <= 8 and g != 32 else 1
     assert _lib.describe_plan(b, g, n, k, m, True, flags).startswith("midbatch")
     for zeros in (zr, None):
-        y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zeros, workspace=None)
+        y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zeros, flags=flags, workspace=None)
         assert need == 0
         zz = z if zeros is not None else np.full_like(z, 128)
         G.assert_close_to_oracle(y, x, o.dequantize(q, s, zz, b, g), f"planes, mid-batch b={b} g={g} M={m}")
         # bit-identical to the pre-sliced tensor: the same codes reach the same arithmetic
         y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zeros, flags=flags).cpu().numpy()
         assert np.array_equal(y, y2)
+
+
+@pytest.mark.parametrize("b,g,m,n", [(4, 128, 8, 304), (2, 128, 5, 304), (3, -1, 7, 304), (6, 128, 6, 304), (8, -1, 8, 304),
+                                     (4, 128, 8, 6144), (8, 128, 7, 6144)])
+def test_gemv_kernel_reads_the_planes_at_five_to_eight_rows(b, g, m, n):
+    # the instantiation for eight batch rows (one or, from 320 row blocks on, two row blocks per
+    # workgroup) on master-resident planes: no workspace, and the result of the pre-sliced tensor
+    k = 1024
+    q, s, z = o.make_layer(n, k, g, seed=b + m)
+    planes = planes_device(q)
+    sc, zr = G.reorder_device(s, n, k, g), G.reorder_device(z, n, k, g)
+    x = o.make_activations(m, k, seed=m)
+    assert _lib.describe_plan(b, g, n, k, m, True).startswith("gemv")
+    for zeros in (zr, None):
+        y, need = gemm_master(b, g, n, k, G.to_dev(x), planes, sc, zeros, workspace=None)
+        assert need == 0
+        zz = z if zeros is not None else np.full_like(z, 128)
+        G.assert_close_to_oracle(y, x, o.dequantize(q, s, zz, b, g), f"planes, gemv b={b} g={g} M={m}")
+        y2 = G.gemm(b, g, n, k, G.to_dev(x), G.pack_device(q, b, True), sc, zeros).cpu().numpy()
+        # (the pre-sliced 2-bit tiles pair their octets differently and the 6- and 8-bit ones multiply their two
+        # code segments apart: another order of the fp32 sums, so close, not identical)
+        assert np.max(np.abs(y.astype(np.float64) - y2)) <= 2.0 ** -9 * np.max(np.abs(y2.astype(np.float64)))
 
 
 @pytest.mark.parametrize("r,mb", [(1, 1), (2, 1), (4, 1), (1, 2), (2, 2), (4, 2), (1, 4), (2, 4), (4, 4)])
