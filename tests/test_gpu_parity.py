@@ -572,9 +572,9 @@ def test_bf16_prefill_weights_are_the_oracles_bit_for_bit(b, zp):
 
 
 @pytest.mark.parametrize("flags", (3, 3 | (64 << 8), 3 | (65 << 8), 3 | (67 << 8), 3 | (72 << 8), 3 | (73 << 8), 3 | (74 << 8),
-                                   3 | (75 << 8)))
+                                   3 | (75 << 8), 3 | (78 << 8), 3 | (79 << 8), 3 | (89 << 8), 3 | (90 << 8)))
 def test_bf16_prefill_large_tiles(flags):
-    # default choice for a large batch, and the ring and largest tiles forced
+    # default choice for a large batch, and the ring, split, mixed and largest tiles forced
     n, k, m, b, g = 2048, 1024, 2048, 4, 128
     q, s16, z16 = o.make_layer(n, k, g, seed=77)
     s = o.round_to_bf16(s16.astype(np.float32))
@@ -586,6 +586,21 @@ def test_bf16_prefill_large_tiles(flags):
     ref = o.linear_f64(x[rows], o.dequantize_bf16(q, s, z, b, g))
     assert np.all(np.isfinite(y))
     assert np.max(np.abs(y[rows] - ref)) <= G.REL_TOL * np.max(np.abs(ref))
+
+
+@pytest.mark.parametrize("b,g,zp", [(4, 32, True), (8, 32, True), (3, -1, False), (6, 128, True), (2, 32, False), (8, -1, True)])
+def test_bf16_64_row_split_tile_every_group_size(b, g, zp):
+    # the 64 x 128 tile with K split in the workgroup on bf16 storage: ragged M and N, seven K tiles
+    n, k, m = 304, 128 * 7, 200
+    q, s16, z16 = o.make_layer(n, k, g, seed=50 + b, symmetric=not zp)
+    s = o.round_to_bf16(s16.astype(np.float32))
+    z = np.round(z16.astype(np.float32))
+    x = o.round_to_bf16(o.make_activations(m, k, seed=b).astype(np.float32))
+    pk = G.pack_device(q, b, True)
+    y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | (89 << 8))
+    ref = o.linear_f64(x, o.dequantize_bf16(q, s, z, b, g))
+    assert np.all(np.isfinite(y))
+    assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref))
 
 
 @pytest.mark.parametrize("b,g,zp", [(4, 128, True), (3, 32, True), (8, 128, False), (2, -1, True), (6, 128, True)])
