@@ -47,7 +47,7 @@ extern "C" {
 #define MATGPTQ_FLAG_ASYNC 1u /* bit 0: 1 = do not synchronise after the launch */
 #define MATGPTQ_FLAG_BF16 2u  /* bit 1: activations / scales / output are bf16 */
 /* Bits 8..17: benchmark-only override of the kernel choice (0 = automatic).  Bits 8..15:
- * 1..42 decode kernel (work split), 64..79, 89 and 90 prefill tile, 80..88 mid-batch kernel (row blocks
+ * 1..42 decode kernel (work split), 64..79, 89 and 90 prefill tile, 80..88 and 91 mid-batch kernel (row blocks
  * and batch rows per workgroup); bits 16..17: decode flavour (1 burst, 2 stream), which also
  * keeps small batches on the decode kernel.  A value that does not apply returns
  * MATGPTQ_EVARIANT. */

@@ -91,7 +91,8 @@ size_t decode_lds_bytes(int R, int S, int W, int kc, int64_t M) {
 // Automatic choice; the flags word can override it for benchmarks:
 //   bits 8..15 : 0 = automatic, 1 + rsel + 3*shape = decode (rsel: R = 1,2,4; shape: kShapes),
 //                64 + cfg = prefill tile configuration 0..15, 89 and 90 = configurations 16 and 17,
-//                80 + rsel + 3*msel = mid-batch kernel (rsel: R = 1,2,4; msel: 16, 32, 64 batch rows)
+//                80 + rsel + 3*msel = mid-batch kernel (rsel: R = 1,2,4; msel: 16, 32, 64 batch rows),
+//                91 = mid-batch kernel with R = 8 and 32 batch rows
 //   bits 16..17: decode flavour, 0 = automatic, 1 = burst, 2 = stream
 int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp, uint32_t flags,
               Plan* p) {
@@ -120,6 +121,8 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   }
   // (four row blocks per mid-batch workgroup only up to 6 bits and one scale per tile: registers)
   const int r_max = group_size == 32 || bits > 6 ? 2 : 4;
+  // (eight: pre-sliced codes up to 4 bits with one scale per tile or row, 32 batch rows per workgroup)
+  const bool eight_rows = group_size != 32 && bits <= 4;
   // row blocks per mid-batch workgroup: as many as still leave about 160 workgroups (the
   // activations are re-read once per workgroup column)
   auto mid_rows = [&](int64_t m_tiles) {
@@ -305,14 +308,19 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
       }
       for (int mb = 2; mb <= (M > 32 ? 4 : 2); mb <<= 1) {
         const int64_t m_tiles = (M + 16 * mb - 1) / (16 * mb);
-        const int r = mid_rows(m_tiles);
+        int r = mid_rows(m_tiles);
+        // Eight row blocks with 32 batch rows (one workgroup per CU) where that still leaves 200
+        // workgroups: the activations are copied half as often (M = 32: 28672 x 4096 21.4 against 21.9 us
+        // at 4 bits, 19.3 against 21.9 at 2; 57344 x 8192 61 against 66, 57 against 65)
+        if (mb == 2 && eight_rows && (int64_t)((row_blocks + 7) / 8) * m_tiles >= 200) r = 8;
         const int64_t wgs = (int64_t)((row_blocks + r - 1) / r) * m_tiles;
         // One workgroup per CU and round.  (With 32 batch rows and at most two row blocks a second
         // one fits, but two together take 1.6 times as long as one: 0.8 of the cost per tile each.)
         // 8-bit codes cost 1.1 times as much per tile, bf16 storage (weights formed in fp32) 1.05
         // times.
         const int64_t slots = 256;
-        const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (mb == 2 && r <= 2 ? 0.8 : 1.0) *
+        // (eight row blocks: 1.3 times the cost their count suggests - 0.41 .. 0.5 us per K tile measured)
+        const double per_tile = 0.85 * (0.12 + 0.016 * r * mb) * (mb == 2 && r <= 2 ? 0.8 : 1.0) * (r == 8 ? 1.3 : 1.0) *
                                 (bits == 8 ? 1.1 : 1.0) * (bf16 ? 1.05 : 1.0);
         const int64_t rounds = (wgs + slots - 1) / slots;
         // (More than a thousand batch rows in more than one round: every XCD then streams most of
@@ -418,8 +426,13 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
   }
   if (variant != 0) {
     if (variant >= 100) return MATGPTQ_EVARIANT;
-    if (variant >= 89) {  // prefill tiles 16 and up
-      if (variant - 89 > 1) return MATGPTQ_EVARIANT;
+    if (variant >= 91) {  // mid-batch kernel, eight row blocks and 32 batch rows per workgroup
+      if (variant > 91 || !eight_rows) return MATGPTQ_EVARIANT;
+      p->decode = false;
+      p->skinny = true;
+      R = 8;
+      p->mb = 2;
+    } else if (variant >= 89) {  // prefill tiles 16 and up
       p->decode = false;
       p->skinny = false;
       p->cfg = variant - 89 + 16;
@@ -449,7 +462,10 @@ int make_plan(int bits, int group_size, int64_t N, int64_t K, int64_t M, bool zp
     // the prefill kernel addresses X through a 32-bit buffer offset
     if ((uint64_t)M * (uint64_t)K * 2u >= (1ull << 32)) return MATGPTQ_ESIZE;
     p->R = p->S = p->W = p->kc = 0;
-    if (p->skinny) p->R = R > r_max ? r_max : R;  // (a forced variant may ask for more)
+    if (p->skinny) {  // (a forced variant may ask for more than the format takes)
+      const int most = eight_rows && p->mb == 2 ? 8 : r_max;
+      p->R = R > most ? most : R;
+    }
     p->stream = false;
     p->smem = 0;
     return MATGPTQ_OK;

@@ -270,6 +270,10 @@ hipError_t launch_rows(const GemmArgs& a, int r, hipStream_t s) {
   // (four row blocks fit the register budget of two waves per SIMD up to 6 bits and with one
   // scale and zero per tile and row block; group 32 carries four; the master planes are eight
   // words per lane from 6 bits on)
+  // (eight row blocks: pre-sliced codes up to 4 bits, 32 batch rows)
+  if constexpr (GROUP != 32 && kBits <= 4 && !MASTER && MB == 2) {
+    if (r >= 8) return launch_r<GROUP, ZP, 8, MB, MASTER>(a, s);
+  }
   if constexpr (GROUP != 32 && kBits <= (MASTER ? 4 : 6)) {
     if (r >= 4) return launch_r<GROUP, ZP, 4, MB, MASTER>(a, s);
   }
@@ -292,7 +296,7 @@ hipError_t launch_storage(const GemmArgs& a, int r, int mb, bool master, hipStre
 
 #define MATGPTQ_CAT2(a, b) a##b
 #define MATGPTQ_CAT(a, b) MATGPTQ_CAT2(a, b)
-// r: row blocks of 16 weight rows per workgroup (1, 2 or 4); mb: blocks of 16 batch rows (1 or 2)
+// r: row blocks of 16 weight rows per workgroup (1, 2, 4 or 8); mb: blocks of 16 batch rows (1, 2 or 4)
 #if MATGPTQ_BF16
 #define MATGPTQ_LAUNCH_NAME MATGPTQ_CAT(MATGPTQ_CAT(launch_skinny_b, MATGPTQ_BITS), _bf16)
 #else

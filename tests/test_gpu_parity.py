@@ -177,6 +177,20 @@ def test_prefill_split_tile_agrees_with_the_plain_tile_closely():
         assert np.mean(y == plain) > 0.9
 
 
+def _mid_variants(b, g):
+    # forced shapes of the mid-batch kernel: 80 + rsel + 3 msel (1, 2, 4 row blocks x 16, 32, 64 batch rows), and
+    # 91 (eight row blocks x 32 batch rows) where the format takes it: up to 4 bits, one scale per tile or row
+    return list(range(80, 89)) + ([91] if b <= 4 and g != 32 else [])
+
+
+def test_midbatch_eight_row_blocks_refused_where_the_format_does_not_take_them():
+    with pytest.raises(_lib.MatGPTQError):
+        _lib.describe_plan(6, 128, 304, 1024, 32, True, 1 | (91 << 8))
+    with pytest.raises(_lib.MatGPTQError):
+        _lib.describe_plan(4, 32, 304, 1024, 32, True, 1 | (91 << 8))
+    assert _lib.describe_plan(4, 128, 304, 1024, 32, True, 1 | (91 << 8)) == "midbatch b4 g128 zp1 R8 mb2"
+
+
 @pytest.mark.parametrize("zp", (False, True))
 @pytest.mark.parametrize("g", GROUPS)
 @pytest.mark.parametrize("b", BITS)
@@ -186,10 +200,10 @@ def test_midbatch_kernel_every_format(b, g, zp):
     n, k, m = 304, 128 * 13, 77
     lay = G.Layer(n, k, b, g, seed=17 * b + (g & 7), zero_points=zp)
     x = o.make_activations(m, k, seed=b + 1)
-    for rsel in range(9):
-        flags = 1 | ((80 + rsel) << 8)
+    for v in _mid_variants(b, g):
+        flags = 1 | (v << 8)
         y = lay.run(x, flags=flags)
-        G.assert_close_to_oracle(y, x, lay.w, f"mid-batch b={b} g={g} zp={zp} rsel={rsel}")
+        G.assert_close_to_oracle(y, x, lay.w, f"mid-batch b={b} g={g} zp={zp} variant={v}")
         assert _lib.describe_plan(b, g, n, k, m, zp, flags).startswith("midbatch")
 
 
@@ -200,9 +214,9 @@ def test_midbatch_kernel_shapes(n, k, m):
     lay = G.Layer(n, k, 4, 128, seed=n + m)
     x = o.make_activations(m, k, seed=m)
     rows = np.r_[0:min(m, 24), max(m - 24, 0):m]
-    for rsel in range(9):
-        y = lay.run(x, flags=1 | ((80 + rsel) << 8))
-        G.assert_close_to_oracle(y[rows], x[rows], lay.w, f"mid-batch {n}x{k} M={m} rsel={rsel}")
+    for v in _mid_variants(4, 128):
+        y = lay.run(x, flags=1 | (v << 8))
+        G.assert_close_to_oracle(y[rows], x[rows], lay.w, f"mid-batch {n}x{k} M={m} variant={v}")
 
 
 def test_midbatch_kernel_agrees_with_prefill_tile_closely():
@@ -221,8 +235,8 @@ def test_midbatch_kernel_agrees_with_prefill_tile_closely():
 def test_midbatch_kernel_outlier_channels():
     lay = G.Layer(512, 4096, 3, 128, seed=12)
     x = o.make_activations(48, 4096, seed=3, outlier_frac=0.01, outlier_gain=20.0)
-    for rsel in range(9):
-        G.assert_close_to_oracle(lay.run(x, flags=1 | ((80 + rsel) << 8)), x, lay.w, f"outliers rsel={rsel}")
+    for v in _mid_variants(3, 128):
+        G.assert_close_to_oracle(lay.run(x, flags=1 | (v << 8)), x, lay.w, f"outliers variant={v}")
 
 
 def test_decode_every_work_split():
@@ -545,10 +559,10 @@ def test_bf16_midbatch_kernel(b, g, zp):
     x = o.round_to_bf16(o.make_activations(m, k, seed=9).astype(np.float32))
     pk = G.pack_device(q, b, True)
     ref = o.linear_f64(x, o.dequantize_bf16(q, s, z, b, g))
-    for rsel in range(9):
-        y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | ((80 + rsel) << 8))
+    for v in _mid_variants(b, g):
+        y = _gemm_bf16(b, g, n, k, x, pk, s, z if zp else None, flags=3 | (v << 8))
         assert np.all(np.isfinite(y))
-        assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref)), (b, g, zp, rsel)
+        assert np.max(np.abs(y - ref)) <= G.REL_TOL * np.max(np.abs(ref)), (b, g, zp, v)
 
 
 @pytest.mark.parametrize("b", (2, 3, 4, 6, 8))

@@ -336,7 +336,17 @@ def test_planner_takes_64_row_split_tiles_where_128_row_ones_leave_half_of_the_c
     # the forced variant: 89
     assert _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 1 | (89 << 8)).endswith("cfg16")
     with pytest.raises(_lib.MatGPTQError):
-        _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 1 | (91 << 8))
+        _lib.describe_plan(4, 128, 8192, 8192, 2048, True, 1 | (92 << 8))
+
+
+def test_planner_gives_eight_row_blocks_to_32_batch_rows_on_layers_with_many_rows():
+    # the mid-batch kernel with eight row blocks and 32 batch rows per workgroup where that leaves 200 workgroups
+    assert _lib.describe_plan(4, 128, 28672, 4096, 32, True) == "midbatch b4 g128 zp1 R8 mb2"
+    assert _lib.describe_plan(2, 128, 28672, 4096, 24, True) == "midbatch b2 g128 zp1 R8 mb2"
+    assert _lib.describe_plan(4, 128, 28672, 4096, 32, True, 3) == "midbatch b4 g128 zp1 R8 mb2"  # bf16 storage
+    assert _lib.describe_plan(4, 128, 10240, 8192, 32, True) == "midbatch b4 g128 zp1 R4 mb2"     # 80 workgroups only
+    assert _lib.describe_plan(6, 128, 28672, 4096, 32, True) == "midbatch b6 g128 zp1 R4 mb2"     # registers
+    assert _lib.describe_plan(4, 128, 28672, 4096, 16, True) == "midbatch b4 g128 zp1 R4 mb1"
 
 
 def test_planner_keeps_group_32_with_zero_points_off_the_largest_ring_tile():
